@@ -1,0 +1,62 @@
+"""ctypes binding of libanyprec_hip.so (the C ABI declared in include/anyprec_hip.h).
+
+There is no fallback: if the library is missing, importing this module raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libanyprec_hip.so")
+
+AP_OK = 0
+AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT = -1, -2, -3, -4, -5, -6
+AP_ABI_VERSION = 1
+
+if not os.path.exists(LIB_PATH):
+    raise ModuleNotFoundError(
+        f"{LIB_PATH} is missing: build it with `python any-precision-llm_amd/build.py` "
+        "(hipcc, --offload-arch=gfx950). There is no CPU fallback."
+    )
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_vp, _ci = ctypes.c_void_p, ctypes.c_int
+lib.ap_abi_version.argtypes = []
+lib.ap_abi_version.restype = _ci
+lib.ap_strerror.argtypes = [_ci]
+lib.ap_strerror.restype = ctypes.c_char_p
+lib.ap_dequant_kbit.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci, _vp]
+lib.ap_dequant_kbit.restype = _ci
+lib.ap_matmul_kbit.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
+lib.ap_matmul_kbit.restype = _ci
+_pi = ctypes.POINTER(ctypes.c_int)
+lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi, _pi]
+lib.ap_matmul_kbit_geometry.restype = _ci
+
+if lib.ap_abi_version() != AP_ABI_VERSION:
+    raise ImportError(
+        f"{LIB_PATH} has ABI version {lib.ap_abi_version()}, this binding needs {AP_ABI_VERSION}: rebuild it"
+    )
+
+EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_geometry")
+
+
+def strerror(code: int) -> str:
+    return lib.ap_strerror(code).decode()
+
+
+def check(code: int, what: str) -> None:
+    """Argument errors -> ValueError, HIP launch errors -> RuntimeError."""
+    if code == AP_OK:
+        return
+    if code < 0:
+        raise ValueError(f"{what}: {strerror(code)} (code {code})")
+    raise RuntimeError(f"{what}: HIP error {code}: {strerror(code)}")
+
+
+def matmul_geometry(M: int, N: int, K: int, w_bits: int) -> dict:
+    vals = [ctypes.c_int() for _ in range(5)]
+    check(lib.ap_matmul_kbit_geometry(M, N, K, w_bits, *[ctypes.byref(v) for v in vals]), "ap_matmul_kbit_geometry")
+    return dict(zip(("wpl", "segments", "groups", "rows", "grid"), (v.value for v in vals)))

@@ -1,0 +1,77 @@
+"""``AnyPrecisionLinear``: counterpart of the reference operator module
+(any_precision/modules/AnyPrecisionLinear.py:10-78) on top of the HIP ops.
+
+Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]``,
+``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
+``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
+Batch dispatch follows the reference (:60-64): more than 8 activation rows ->
+``dequant_kbit`` + ``torch.matmul``, otherwise ``matmul_kbit``.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+try:
+    from any_precision_ext import matmul_kbit, dequant_kbit
+except ModuleNotFoundError:
+    matmul_kbit, dequant_kbit = None, None
+
+
+class AnyPrecisionLinear(nn.Module):
+    def __init__(self, in_features, out_features, supported_bits, bias=True, precisions=None, device=None,
+                 dtype=None):
+        super().__init__()
+        if dequant_kbit is None or matmul_kbit is None:
+            raise ModuleNotFoundError("libanyprec_hip.so is not built: run `python any-precision-llm_amd/build.py`.")
+        if precisions is None:
+            precisions = supported_bits
+        if not isinstance(precisions, list):
+            raise RuntimeError("supported_bits must be a list of integers.")
+        if dtype is not None and dtype != torch.float16:
+            raise RuntimeError("Only float16 is supported for now.")
+        if in_features % 32 != 0:
+            raise RuntimeError("in_features must be a multiple of 32.")
+
+        self.in_features = in_features
+        self.out_features = out_features
+        self.precisions = precisions
+        self.precision = max(self.precisions)
+        self.supported_bits = supported_bits
+
+        self.register_buffer(
+            "qweight",
+            torch.empty((max(supported_bits), out_features, in_features // 32), dtype=torch.int32, device=device),
+        )
+        for bit in supported_bits:
+            self.register_buffer(f"lut{bit}", torch.empty((out_features, 2 ** bit), dtype=dtype, device=device))
+        if bias:
+            self.register_buffer("bias", torch.empty((out_features,), dtype=dtype, device=device))
+        else:
+            self.bias = None
+
+    def prune_precisions(self):
+        self.qweight = self.qweight[:max(self.precisions)]
+        for bit in self.supported_bits:
+            if bit not in self.precisions:
+                delattr(self, f"lut{bit}")
+
+    def forward(self, x, **kwargs):
+        w_bits = kwargs["precision"] if "precision" in kwargs else self.precision
+        lut = self._buffers[f"lut{w_bits}"]
+        if x.numel() // x.shape[-1] > 8:
+            weight = dequant_kbit(self.qweight, lut, w_bits)
+            x = torch.matmul(x, weight.T)
+        else:
+            x = matmul_kbit(x, self.qweight, lut, w_bits)
+        if self.bias is not None:
+            x += self.bias
+        return x
+
+    def set_precision(self, precision):
+        if precision not in self.precisions:
+            raise RuntimeError(f"{self.precisions}-bit precisions are supported but {precision}-bit was specified.")
+        self.precision = precision
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"

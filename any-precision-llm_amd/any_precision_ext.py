@@ -1,0 +1,80 @@
+"""Drop-in replacement for the reference's native module ``any_precision_ext``
+(any_precision/modules/kernels/main.cu:145-148): same op names, same positional
+signatures, same result shapes and dtypes.
+
+    matmul_kbit(in, qweight, lut, w_bits) -> Tensor   main.cu:93-143
+    dequant_kbit(qweight, lut, w_bits)    -> Tensor   main.cu:60-91
+
+The ops validate their arguments, allocate the result with torch and hand raw
+device pointers plus torch's current HIP stream to libanyprec_hip.so.  Where
+the reference asserts (compiled out in release builds) or exits the process,
+these raise ``ValueError`` / ``RuntimeError``.  Launches go to the *current*
+stream (the reference uses the legacy default stream, main.cu:83,134), so the
+ops can be captured into HIP graphs.
+"""
+from __future__ import annotations
+
+import torch
+
+from any_precision_amd import _capi
+
+__all__ = ["matmul_kbit", "dequant_kbit"]
+
+_lib = _capi.lib
+
+
+def _check_weight(qweight: torch.Tensor, lut: torch.Tensor, w_bits: int, op: str):
+    if not isinstance(w_bits, int) or isinstance(w_bits, bool):
+        raise TypeError(f"{op}: w_bits must be an int, got {type(w_bits).__name__}")
+    if w_bits < 3 or w_bits > 8:
+        raise ValueError(f"{op}: w_bits must be in 3..8, got {w_bits}")
+    if qweight.dim() != 3 or qweight.dtype != torch.int32:
+        raise ValueError(f"{op}: qweight must be a 3-D int32 tensor [planes, N, K/32], got "
+                         f"{tuple(qweight.shape)} {qweight.dtype}")
+    if lut.dtype != torch.float16:
+        raise ValueError(f"{op}: lut must be float16, got {lut.dtype}")
+    if not qweight.is_cuda or qweight.device != lut.device:
+        raise ValueError(f"{op}: qweight and lut must live on the same GPU, got {qweight.device} and {lut.device}")
+    planes, N, W = qweight.shape
+    if planes < w_bits:
+        raise ValueError(f"{op}: qweight holds {planes} planes, w_bits={w_bits} needs {w_bits}")
+    if N < 1 or W < 1:
+        raise ValueError(f"{op}: empty weight {tuple(qweight.shape)}")
+    if tuple(lut.shape) != (N, 1 << w_bits):
+        raise ValueError(f"{op}: lut must be [{N}, {1 << w_bits}] for w_bits={w_bits}, got {tuple(lut.shape)}")
+    if not qweight.is_contiguous() or not lut.is_contiguous():
+        raise ValueError(f"{op}: qweight and lut must be contiguous")
+    return N, W * 32
+
+
+def dequant_kbit(qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:
+    """fp16 [N, K] with out[n, k] = lut[n, code[n, k] >> (P - w_bits)]."""
+    N, K = _check_weight(qweight, lut, w_bits, "dequant_kbit")
+    with torch.cuda.device(qweight.device):
+        out = torch.empty((N, K), dtype=torch.float16, device=qweight.device)
+        rc = _lib.ap_dequant_kbit(qweight.data_ptr(), lut.data_ptr(), out.data_ptr(), N, K, w_bits,
+                                  torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "dequant_kbit")
+    return out
+
+
+def matmul_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:
+    """fp16 in_.shape[:-1] + [N]; M = in_.numel() // K must be in 1..8 (main.cu:108)."""
+    N, K = _check_weight(qweight, lut, w_bits, "matmul_kbit")
+    if in_.dtype != torch.float16:
+        raise ValueError(f"matmul_kbit: input must be float16, got {in_.dtype}")
+    if in_.device != qweight.device:
+        raise ValueError(f"matmul_kbit: input on {in_.device}, weight on {qweight.device}")
+    if in_.dim() < 1 or in_.shape[-1] != K:
+        raise ValueError(f"matmul_kbit: input last dim must be K={K}, got {tuple(in_.shape)}")
+    M = in_.numel() // K
+    if M < 1 or M > 8:
+        raise ValueError(f"matmul_kbit: batch M={M} outside 1..8; use dequant_kbit + matmul for larger batches")
+    if not in_.is_contiguous():
+        raise ValueError("matmul_kbit: input must be contiguous")
+    with torch.cuda.device(qweight.device):
+        out = torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device)
+        rc = _lib.ap_matmul_kbit(in_.data_ptr(), qweight.data_ptr(), lut.data_ptr(), out.data_ptr(), M, N, K,
+                                 w_bits, torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "matmul_kbit")
+    return out

@@ -1,0 +1,191 @@
+// C ABI of libanyprec_hip: argument checks, launch geometry, dispatch.
+// The declarations and their reference counterparts are in include/anyprec_hip.h.
+#include <hip/hip_runtime.h>
+#include <stdlib.h>
+
+#include "anyprec_hip.h"
+#include "ap_dequant.hpp"
+#include "ap_gemv.hpp"
+
+namespace {
+
+using namespace ap;
+
+constexpr int kNumCUs = 256;  // MI355X: 8 XCDs x 32 CUs
+
+struct Tuning {
+    int target_waves;  // waves the GEMV grid aims for (rows per wave follows)
+    int force_rows;    // > 0: rows per wave, overrides target_waves
+    int force_wpl;     // > 0: words per lane
+    int dequant_blocks_per_cu;
+};
+
+int env_int(const char *name, int dflt) {
+    const char *v = getenv(name);
+    return (v && *v) ? atoi(v) : dflt;
+}
+
+const Tuning &tuning() {
+    static const Tuning t = {
+        env_int("AP_GEMV_TARGET_WAVES", 4096),
+        env_int("AP_GEMV_ROWS", 0),
+        env_int("AP_GEMV_WPL", 0),
+        env_int("AP_DEQUANT_BLOCKS_PER_CU", 8),
+    };
+    return t;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_common(int N, int K, int w_bits) {
+    if (w_bits < 3 || w_bits > 8) return AP_EBITS;
+    if (N < 1 || K < 32 || (K & 31) != 0) return AP_ESHAPE;
+    return AP_OK;
+}
+
+struct GemvGeometry {
+    int wpl, S, G, R, grid;
+};
+
+int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
+    const int rc = check_common(N, K, w_bits);
+    if (rc != AP_OK) return rc;
+    if (M < 1 || M > 8) return AP_EBATCH;
+    const Tuning &t = tuning();
+    const int W = K >> 5;
+    int wpl = (M <= 2 && (W & 1) == 0) ? 2 : 1;
+    if (t.force_wpl == 1 || (t.force_wpl == 2 && (W & 1) == 0 && M <= 2)) wpl = t.force_wpl;
+    const int seg = kWave * wpl;
+    const int S = (W + seg - 1) / seg;
+    if (S > kGemvMaxWaves) return AP_ELIMIT;
+    const int G = S >= 4 ? 1 : (S == 3 ? 1 : 4 / S);
+    int R = t.force_rows > 0 ? t.force_rows : (int)(((long long)N * S + t.target_waves - 1) / t.target_waves);
+    if (R < 1) R = 1;
+    if (R > kGemvMaxRows) R = kGemvMaxRows;
+    geo->wpl = wpl;
+    geo->S = S;
+    geo->G = G;
+    geo->R = R;
+    geo->grid = (N + G * R - 1) / (G * R);
+    return AP_OK;
+}
+
+template <int BITS, int M, int WPL>
+void launch_gemv(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                 uint16_t *out, int N, int K, hipStream_t stream) {
+    const dim3 block(kWave, geo.S, geo.G);
+    gemv_kbit_kernel<BITS, M, WPL><<<dim3(geo.grid), block, 0, stream>>>(
+        reinterpret_cast<const half_t *>(x), qweight, reinterpret_cast<const half_t *>(lut),
+        reinterpret_cast<half_t *>(out), N, K, geo.R);
+}
+
+template <int BITS, int M>
+void launch_gemv_wpl(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                     uint16_t *out, int N, int K, hipStream_t stream) {
+    if constexpr (M <= 2) {
+        if (geo.wpl == 2) return launch_gemv<BITS, M, 2>(geo, x, qweight, lut, out, N, K, stream);
+    }
+    launch_gemv<BITS, M, 1>(geo, x, qweight, lut, out, N, K, stream);
+}
+
+template <int BITS>
+void launch_gemv_m(int M, const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight,
+                   const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream) {
+    switch (M) {
+        case 1: return launch_gemv_wpl<BITS, 1>(geo, x, qweight, lut, out, N, K, stream);
+        case 2: return launch_gemv_wpl<BITS, 2>(geo, x, qweight, lut, out, N, K, stream);
+        case 3: return launch_gemv_wpl<BITS, 3>(geo, x, qweight, lut, out, N, K, stream);
+        case 4: return launch_gemv_wpl<BITS, 4>(geo, x, qweight, lut, out, N, K, stream);
+        case 5: return launch_gemv_wpl<BITS, 5>(geo, x, qweight, lut, out, N, K, stream);
+        case 6: return launch_gemv_wpl<BITS, 6>(geo, x, qweight, lut, out, N, K, stream);
+        case 7: return launch_gemv_wpl<BITS, 7>(geo, x, qweight, lut, out, N, K, stream);
+        default: return launch_gemv_wpl<BITS, 8>(geo, x, qweight, lut, out, N, K, stream);
+    }
+}
+
+template <int BITS>
+void launch_dequant(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream) {
+    int blocks = (N + kDequantWaves - 1) / kDequantWaves;
+    const int cap = kNumCUs * tuning().dequant_blocks_per_cu;
+    if (blocks > cap) blocks = cap;
+    dequant_kbit_kernel<BITS><<<dim3(blocks), dim3(kDequantWaves * kWave), 0, stream>>>(
+        qweight, reinterpret_cast<const half_t *>(lut), reinterpret_cast<half_t *>(out), N, K);
+}
+
+int launch_status() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? AP_OK : (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ap_abi_version(void) { return AP_ABI_VERSION; }
+
+const char *ap_strerror(int code) {
+    switch (code) {
+        case AP_OK: return "ok";
+        case AP_ENULL: return "null pointer argument";
+        case AP_EBITS: return "w_bits must be in 3..8";
+        case AP_ESHAPE: return "need N >= 1 and K a positive multiple of 32";
+        case AP_EALIGN: return "pointer not 16-byte aligned";
+        case AP_EBATCH: return "batch M outside the range this entry point serves";
+        case AP_ELIMIT: return "size exceeds the launch geometry limits";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error code";
+}
+
+int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, int w_bits,
+                    void *stream) {
+    if (!qweight || !lut || !out) return AP_ENULL;
+    const int rc = check_common(N, K, w_bits);
+    if (rc != AP_OK) return rc;
+    if (!aligned16(qweight) || !aligned16(lut) || !aligned16(out)) return AP_EALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (w_bits) {
+        case 3: launch_dequant<3>(qweight, lut, out, N, K, st); break;
+        case 4: launch_dequant<4>(qweight, lut, out, N, K, st); break;
+        case 5: launch_dequant<5>(qweight, lut, out, N, K, st); break;
+        case 6: launch_dequant<6>(qweight, lut, out, N, K, st); break;
+        case 7: launch_dequant<7>(qweight, lut, out, N, K, st); break;
+        default: launch_dequant<8>(qweight, lut, out, N, K, st); break;
+    }
+    return launch_status();
+}
+
+int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segments, int *groups, int *rows,
+                            int *grid) {
+    GemvGeometry geo;
+    const int rc = gemv_geometry(M, N, K, w_bits, &geo);
+    if (rc != AP_OK) return rc;
+    if (wpl) *wpl = geo.wpl;
+    if (segments) *segments = geo.S;
+    if (groups) *groups = geo.G;
+    if (rows) *rows = geo.R;
+    if (grid) *grid = geo.grid;
+    return AP_OK;
+}
+
+int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N,
+                   int K, int w_bits, void *stream) {
+    if (!x || !qweight || !lut || !out) return AP_ENULL;
+    GemvGeometry geo;
+    const int rc = gemv_geometry(M, N, K, w_bits, &geo);
+    if (rc != AP_OK) return rc;
+    if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (w_bits) {
+        case 3: launch_gemv_m<3>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 4: launch_gemv_m<4>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 5: launch_gemv_m<5>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 6: launch_gemv_m<6>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 7: launch_gemv_m<7>(M, geo, x, qweight, lut, out, N, K, st); break;
+        default: launch_gemv_m<8>(M, geo, x, qweight, lut, out, N, K, st); break;
+    }
+    return launch_status();
+}
+
+}  // extern "C"

@@ -1,0 +1,65 @@
+// Bitplane dequantiser for gfx950: out[n,k] = lut[n, index_b(n,k)], fp16 [N,K].
+//
+// Replaces the reference's dequant_kbit_store<bits>
+// (any_precision/modules/kernels/dequant.cuh:177-242).  Result is a pure
+// table copy, hence bit-exact by construction when the index is right.
+//
+// Mapping: one wave64 per row at a time; lane l owns word l, l+64, ... of the
+// row.  Per word a lane reads one dword per plane (a wave covers 256 B of each
+// plane, fully coalesced), rebuilds its 32 indices in registers, gathers from
+// the row's table in LDS and emits four 16-byte stores; for a fixed byte
+// group the 32 lanes of a chunk write 512 contiguous bytes.
+#pragma once
+#include "ap_bitplane.hpp"
+#include "ap_device.hpp"
+
+namespace ap {
+
+constexpr int kDequantWaves = 4;  // waves per workgroup
+
+template <int BITS>
+__global__ __launch_bounds__(kDequantWaves * kWave) void dequant_kbit_kernel(
+    const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
+    half_t *__restrict__ out, int N, int K) {
+    constexpr int NC = 1 << BITS;
+    __shared__ __attribute__((aligned(16))) half_t tables[kDequantWaves][2][NC];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    const int W = K >> 5;
+    const int wave_stride = gridDim.x * kDequantWaves;
+    const size_t plane_stride = (size_t)N * W;
+
+    int buf = 0;
+    for (int row = blockIdx.x * kDequantWaves + wave; row < N; row += wave_stride, buf ^= 1) {
+        half_t *tab = tables[wave][buf];
+        lut_stage<BITS>(lut_fetch<BITS>(lut + (size_t)row * NC, lane), tab, lane);
+        // LDS operations of one wave complete in order, so the table is
+        // visible to the gathers below without a workgroup barrier.
+        __builtin_amdgcn_wave_barrier();
+
+        const uint32_t *wrow = qweight + (size_t)row * W;
+        half_t *orow = out + (size_t)row * K;
+        for (int w = lane; w < W; w += kWave) {
+            uint32_t q[BITS];
+#pragma unroll
+            for (int p = 0; p < BITS; p++) q[p] = wrow[p * plane_stride + w];
+            uint32_t idx[8];
+            planes_to_indices<BITS>(q, idx);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int sh = 8 * (3 - j);
+                u32x4 v;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const uint16_t lo = __builtin_bit_cast(uint16_t, tab[(idx[2 * i] >> sh) & 0xffu]);
+                    const uint16_t hi = __builtin_bit_cast(uint16_t, tab[(idx[2 * i + 1] >> sh) & 0xffu]);
+                    v[i] = (uint32_t)lo | ((uint32_t)hi << 16);
+                }
+                *reinterpret_cast<u32x4 *>(orow + group_base(w, j, K)) = v;
+            }
+        }
+    }
+}
+
+}  // namespace ap

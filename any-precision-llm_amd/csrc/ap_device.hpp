@@ -1,0 +1,76 @@
+// Device-side helpers shared by the gfx950 kernels: vector types, wave64
+// reductions through DPP, LUT staging into LDS.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ap {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+// fp32 += a.x*b.x + a.y*b.y  (v_dot2c_f32_f16: fp16 products, fp32 accumulate)
+__device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w), __builtin_bit_cast(half2_t, x), acc, false);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over the 64 lanes of a wave; the total is returned in every lane.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);  // row_half_mirror: lanes 0-3 <-> 7-4 within 8
+    v = dpp_add<0x140>(v);  // row_mirror: 0-7 <-> 15-8 within a row of 16
+    // every lane of a 16-lane row now holds its row's sum
+    const int vi = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// Copy one row's table of 2^BITS fp16 entries from global memory into this
+// wave's LDS slot.  Split in two so the global load can be issued early.
+template <int BITS>
+struct LutRegs {
+    u32x2 v;
+};
+
+template <int BITS>
+__device__ __forceinline__ LutRegs<BITS> lut_fetch(const half_t *lut_row, int lane) {
+    LutRegs<BITS> r;
+    r.v = u32x2{0u, 0u};
+    constexpr int dwords = (1 << BITS) / 2;          // table size in dwords
+    if constexpr (dwords >= 128) {                   // 8 bits: 64 lanes x 8 B
+        r.v = reinterpret_cast<const u32x2 *>(lut_row)[lane];
+    } else if constexpr (dwords == 64) {             // 7 bits: 64 lanes x 4 B
+        r.v.x = reinterpret_cast<const uint32_t *>(lut_row)[lane];
+    } else {                                         // <= 6 bits: first `dwords` lanes
+        if (lane < dwords) r.v.x = reinterpret_cast<const uint32_t *>(lut_row)[lane];
+    }
+    return r;
+}
+
+template <int BITS>
+__device__ __forceinline__ void lut_stage(const LutRegs<BITS> &r, half_t *slot, int lane) {
+    constexpr int dwords = (1 << BITS) / 2;
+    if constexpr (dwords >= 128) {
+        reinterpret_cast<u32x2 *>(slot)[lane] = r.v;
+    } else if constexpr (dwords == 64) {
+        reinterpret_cast<uint32_t *>(slot)[lane] = r.v.x;
+    } else {
+        if (lane < dwords) reinterpret_cast<uint32_t *>(slot)[lane] = r.v.x;
+    }
+}
+
+}  // namespace ap

@@ -1,0 +1,42 @@
+// Host build of the pure-integer device helpers, for the CPU unit tests.
+// Compiled with g++ into libanyprec_hostcheck.so; exports the in-lane plane ->
+// index transposes and the layout address helpers exactly as the kernels use them.
+#include "ap_bitplane.hpp"
+
+extern "C" {
+
+int aph_planes_to_indices(const uint32_t *q, int bits, int shift, uint32_t *idx) {
+    uint32_t out[8];
+#define AP_CASE(B, S)                                        \
+    if (bits == B && shift == S) {                           \
+        uint32_t qq[B];                                      \
+        for (int i = 0; i < B; i++) qq[i] = q[i];            \
+        ap::planes_to_indices<B, S>(qq, out);                \
+        for (int i = 0; i < 8; i++) idx[i] = out[i];         \
+        return 0;                                            \
+    }
+    AP_CASE(1, 0) AP_CASE(2, 0) AP_CASE(3, 0) AP_CASE(4, 0) AP_CASE(5, 0) AP_CASE(6, 0) AP_CASE(7, 0) AP_CASE(8, 0)
+    AP_CASE(3, 1) AP_CASE(4, 1) AP_CASE(5, 1) AP_CASE(6, 1) AP_CASE(7, 1)
+#undef AP_CASE
+    return -1;
+}
+
+int aph_planes_to_pair_indices(const uint32_t *q, int bits, uint32_t *pidx) {
+    uint32_t out[4];
+    if (bits == 3) {
+        uint32_t qq[3] = {q[0], q[1], q[2]};
+        ap::planes_to_pair_indices<3>(qq, out);
+    } else if (bits == 4) {
+        uint32_t qq[4] = {q[0], q[1], q[2], q[3]};
+        ap::planes_to_pair_indices<4>(qq, out);
+    } else {
+        return -1;
+    }
+    for (int i = 0; i < 4; i++) pidx[i] = out[i];
+    return 0;
+}
+
+int aph_chunk_words(int w, int K) { return ap::chunk_words(w, K); }
+int aph_group_base(int w, int j, int K) { return ap::group_base(w, j, K); }
+
+}  // extern "C"

@@ -1,0 +1,71 @@
+/*
+ * libanyprec_hip -- C ABI of the MI355X (gfx950) any-precision bitplane kernels.
+ *
+ * Drop-in boundary for the reference's native ops module `any_precision_ext`
+ * (any_precision/modules/kernels/main.cu).  Plain pointers and sizes only; all
+ * pointers are device pointers on the current HIP device, all buffers are
+ * owned by the caller, nothing is allocated or synchronised inside, and every
+ * launch goes to the stream that is passed in (NULL = default stream).
+ *
+ * Data formats (identical to the reference checkpoint format):
+ *   qweight  uint32 [planes >= w_bits, N, K/32], contiguous; bit pattern of the
+ *            int32 tensor written by any_precision/quantization/pack.py:90-99.
+ *            Plane 0 is the MSB of the parent code; only planes 0..w_bits-1
+ *            are read.
+ *   lut      fp16 [N, 2^w_bits], the table for that w_bits
+ *            (any_precision/modules/AnyPrecisionLinear.py:34-38).
+ *   x        fp16 [M, K] row-major;  out fp16 [M, N] (matmul) or [N, K] (dequant).
+ *
+ * Return value: AP_OK (0), a negative AP_E* argument error, or a positive
+ * hipError_t from the launch.  The library never exits the process (the
+ * reference prints and calls exit(), main.cu:5-12).
+ */
+#ifndef ANYPREC_HIP_H
+#define ANYPREC_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AP_ABI_VERSION 1
+
+enum {
+    AP_OK = 0,
+    AP_ENULL = -1,   /* a required pointer is NULL                          */
+    AP_EBITS = -2,   /* w_bits outside 3..8 (main.cu:70,108)                */
+    AP_ESHAPE = -3,  /* N < 1, K < 32 or K not a multiple of 32 (pack.py:15) */
+    AP_EALIGN = -4,  /* a pointer is not 16-byte aligned                    */
+    AP_EBATCH = -5,  /* M outside the range the entry point serves          */
+    AP_ELIMIT = -6   /* a size exceeds what the launch geometry can express */
+};
+
+/* Replaces dequant_kbit(qweight, lut, w_bits) -> Tensor[N,K]
+ * (main.cu:60-91, kernel dequant.cuh:177-242).
+ * out[n,k] = lut[n, code[n,k] >> (P - w_bits)], bit-exact copy of table entries. */
+int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
+                    int N, int K, int w_bits, void *stream);
+
+/* Replaces matmul_kbit(in, qweight, lut, w_bits) -> Tensor[..., N]
+ * (main.cu:93-143, kernel matmul.cuh:16-167).  1 <= M <= 8 as in the
+ * reference (main.cu:108).  fp32 accumulation, fp16 result. */
+int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                   uint16_t *out, int M, int N, int K, int w_bits, void *stream);
+
+/* Human-readable text for a return code of the functions above. */
+const char *ap_strerror(int code);
+
+/* AP_ABI_VERSION the library was built with. */
+int ap_abi_version(void);
+
+/* Launch geometry the GEMV would use, for reports and tests: words per lane,
+ * K-segments per workgroup, row groups per workgroup, rows per wave, grid size.
+ * Returns AP_OK or the same argument errors as ap_matmul_kbit. */
+int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits,
+                            int *wpl, int *segments, int *groups, int *rows, int *grid);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ANYPREC_HIP_H */

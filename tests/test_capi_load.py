@@ -1,0 +1,75 @@
+"""The C-ABI library loads and exports every function include/*.h declares
+(CPU only: no compute entry point is launched here)."""
+import ctypes
+import glob
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "any-precision-llm_amd", "lib", "libanyprec_hip.so")
+
+
+def _declared_functions():
+    names = []
+    for hdr in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(hdr).read(), flags=re.S)
+        names += re.findall(r"\b(ap_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_boundary():
+    names = _declared_functions()
+    for must in ("ap_dequant_kbit", "ap_matmul_kbit", "ap_strerror", "ap_abi_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    assert os.path.exists(LIB), "build libanyprec_hip.so first (python any-precision-llm_amd/build.py)"
+    lib = ctypes.CDLL(LIB)
+    for name in _declared_functions():
+        assert hasattr(lib, name), name
+
+
+def test_binding_lists_every_declared_symbol():
+    from any_precision_amd import _capi
+    assert sorted(_capi.EXPORTS) == _declared_functions()
+    assert _capi.lib.ap_abi_version() == _capi.AP_ABI_VERSION
+
+
+def test_strerror_and_argument_errors_need_no_gpu():
+    from any_precision_amd import _capi
+    L = _capi.lib
+    assert _capi.strerror(0) == "ok"
+    for code in (-1, -2, -3, -4, -5, -6):
+        assert _capi.strerror(code) not in ("ok", "unknown error code")
+    fake = 4096  # non-null, 16-byte aligned; argument errors return before any launch
+    assert L.ap_dequant_kbit(None, fake, fake, 4, 64, 3, None) == _capi.AP_ENULL
+    assert L.ap_dequant_kbit(fake, fake, fake, 4, 64, 2, None) == _capi.AP_EBITS
+    assert L.ap_dequant_kbit(fake, fake, fake, 4, 64, 9, None) == _capi.AP_EBITS
+    assert L.ap_dequant_kbit(fake, fake, fake, 4, 48, 3, None) == _capi.AP_ESHAPE
+    assert L.ap_dequant_kbit(fake, fake, fake, 0, 64, 3, None) == _capi.AP_ESHAPE
+    assert L.ap_dequant_kbit(fake, fake, fake + 8, 4, 64, 3, None) == _capi.AP_EALIGN
+    assert L.ap_matmul_kbit(fake, fake, fake, None, 1, 4, 64, 3, None) == _capi.AP_ENULL
+    assert L.ap_matmul_kbit(fake, fake, fake, fake, 0, 4, 64, 3, None) == _capi.AP_EBATCH
+    assert L.ap_matmul_kbit(fake, fake, fake, fake, 9, 4, 64, 3, None) == _capi.AP_EBATCH
+    assert L.ap_matmul_kbit(fake + 2, fake, fake, fake, 1, 4, 64, 3, None) == _capi.AP_EALIGN
+    assert L.ap_matmul_kbit(fake, fake, fake, fake, 1, 4, 64, 11, None) == _capi.AP_EBITS
+    with pytest.raises(ValueError):
+        _capi.check(_capi.AP_EBITS, "x")
+    with pytest.raises(RuntimeError):
+        _capi.check(98, "x")
+
+
+def test_geometry_covers_rows_and_words():
+    from any_precision_amd import _capi
+    for M in (1, 2, 4, 8):
+        for N, K in ((4096, 4096), (11008, 4096), (4096, 11008), (1024, 4096), (4096, 14336), (7, 32), (5, 2080)):
+            g = _capi.matmul_geometry(M, N, K, 4)
+            W = K // 32
+            assert g["segments"] * 64 * g["wpl"] >= W and W % g["wpl"] == 0
+            assert g["segments"] * g["groups"] <= 16 and 1 <= g["rows"] <= 8
+            assert g["grid"] * g["groups"] * g["rows"] >= N
+    with pytest.raises(ValueError):
+        _capi.matmul_geometry(1, 4, 32 * 64 * 2 * 17, 4)     # more K-segments than a workgroup holds

@@ -1,0 +1,48 @@
+"""Argument validation of the drop-in ops (CPU only: every case raises before a launch)."""
+import pytest
+import torch
+
+import any_precision_ext as ext
+
+
+def _w(planes=8, N=4, W=2, b=3):
+    return torch.zeros((planes, N, W), dtype=torch.int32), torch.zeros((N, 1 << b), dtype=torch.float16)
+
+
+def test_op_names_and_signatures():
+    import inspect
+    assert list(inspect.signature(ext.matmul_kbit).parameters)[1:] == ["qweight", "lut", "w_bits"]
+    assert list(inspect.signature(ext.dequant_kbit).parameters) == ["qweight", "lut", "w_bits"]
+
+
+@pytest.mark.parametrize("bits", [0, 2, 9, -1])
+def test_w_bits_range(bits):
+    q, l = _w()
+    with pytest.raises(ValueError, match="w_bits"):
+        ext.dequant_kbit(q, l, bits)
+    with pytest.raises(ValueError, match="w_bits"):
+        ext.matmul_kbit(torch.zeros(1, 64, dtype=torch.float16), q, l, bits)
+
+
+def test_w_bits_type():
+    q, l = _w()
+    with pytest.raises(TypeError):
+        ext.dequant_kbit(q, l, 3.0)
+
+
+def test_dtypes_and_dims():
+    q, l = _w()
+    with pytest.raises(ValueError, match="int32"):
+        ext.dequant_kbit(q.to(torch.int64), l, 3)
+    with pytest.raises(ValueError, match="3-D"):
+        ext.dequant_kbit(q[0], l, 3)
+    with pytest.raises(ValueError, match="float16"):
+        ext.dequant_kbit(q, l.float(), 3)
+
+
+def test_cpu_tensors_are_rejected_not_computed():
+    q, l = _w()
+    with pytest.raises(ValueError, match="GPU"):
+        ext.dequant_kbit(q, l, 3)
+    with pytest.raises(ValueError, match="GPU"):
+        ext.matmul_kbit(torch.zeros(1, 64, dtype=torch.float16), q, l, 3)

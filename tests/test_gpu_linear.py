@@ -1,0 +1,68 @@
+"""AnyPrecisionLinear on the GPU: state-dict format, precision switching, both batch branches."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_close_gemv, make
+from any_precision_amd import packing, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _module(L, bias=True, precisions=None):
+    from any_precision_amd import AnyPrecisionLinear
+    bits = list(range(L.seed_bits, L.parent_bits + 1))
+    m = AnyPrecisionLinear(L.K, L.N, bits, bias=bias, precisions=precisions, device="cuda", dtype=torch.float16)
+    sd = {k: torch.from_numpy(v) for k, v in packing.pack_layer(L.codes, L.luts).items()}
+    if bias:
+        sd["bias"] = torch.from_numpy(np.linspace(-1, 1, L.N).astype(np.float16))
+    m.load_state_dict(sd)
+    return m, sd
+
+
+def test_state_dict_keys_shapes_dtypes():
+    L = make(64, 1056, seed=0)
+    m, _ = _module(L)
+    sd = m.state_dict()
+    assert sorted(sd) == sorted(["qweight", "bias"] + [f"lut{b}" for b in range(3, 9)])
+    assert sd["qweight"].shape == (8, 64, 33) and sd["qweight"].dtype == torch.int32
+    for b in range(3, 9):
+        assert sd[f"lut{b}"].shape == (64, 1 << b) and sd[f"lut{b}"].dtype == torch.float16
+    assert m.precision == 8 and m.precisions == list(range(3, 9))
+
+
+def test_forward_both_branches_and_bias(oracle):
+    L = make(128, 4096, seed=1)
+    m, sd = _module(L)
+    bias = sd["bias"].numpy().astype(np.float64)
+    for b in (3, 5, 8):
+        for M in (1, 8, 9, 40):
+            x = synth.make_x(M, L.K, seed=M)
+            y = m(torch.from_numpy(x).cuda(), precision=b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert y.shape == (M, L.N)
+            assert_close_gemv(y, want + bias, f"b={b} M={M}")
+
+
+def test_set_precision_and_prune(oracle):
+    L = make(32, 1024, seed=2)
+    m, _ = _module(L, bias=False, precisions=[3, 4, 6])
+    assert m.precision == 6
+    with pytest.raises(RuntimeError):
+        m.set_precision(8)
+    m.prune_precisions()
+    assert m.qweight.shape[0] == 6
+    assert not hasattr(m, "lut8") and not hasattr(m, "lut5") and hasattr(m, "lut4")
+    x = synth.make_x(2, L.K)
+    for b in (3, 4, 6):
+        m.set_precision(b)
+        _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+        assert_close_gemv(m(torch.from_numpy(x).cuda()), want, f"b={b}")
+
+
+def test_constructor_errors():
+    from any_precision_amd import AnyPrecisionLinear
+    with pytest.raises(RuntimeError):
+        AnyPrecisionLinear(64, 8, [3, 4], dtype=torch.float32)
+    with pytest.raises(RuntimeError):
+        AnyPrecisionLinear(64, 8, [3, 4], precisions=(3, 4))

@@ -1,0 +1,149 @@
+"""matmul_kbit on the GPU against the oracle, through the C ABI.
+
+Tolerance: 1e-2 relative (normwise and against max |y|), fp32 accumulate / fp16 out
+on the GPU against double accumulate / one rounding in the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_bit_exact, assert_close_gemv, layer_to_gpu, make
+from any_precision_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+RAGGED = [(1, 32), (7, 32), (5, 96), (13, 1056), (4, 2080), (130, 992), (33, 1024), (3, 3104), (21, 4128)]
+FULL = [(4096, 4096), (11008, 4096), (4096, 11008), (1024, 4096), (14336, 4096), (4096, 14336)]
+SLICES = [(256, 4096), (192, 11008), (160, 14336)]
+
+
+@pytest.fixture(scope="module")
+def ext():
+    import any_precision_ext
+    return any_precision_ext
+
+
+def _x(M, K, seed=0):
+    x = synth.make_x(M, K, seed)
+    return x, torch.from_numpy(x).cuda()
+
+
+@pytest.mark.parametrize("N,K", RAGGED)
+def test_ragged_shapes_all_bits_all_batches(ext, oracle, N, K):
+    L = make(N, K, seed=N + K)
+    q, luts = layer_to_gpu(L)
+    for b in range(3, 9):
+        for M in range(1, 9):
+            print(f"gemv N={N} K={K} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            got = ext.matmul_kbit(xg, q, luts[b], b)
+            assert got.shape == (M, N) and got.dtype == torch.float16
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+
+
+@pytest.mark.parametrize("N,K", SLICES)
+def test_row_slices_of_benchmark_shapes_all_batches(ext, oracle, N, K):
+    L = make(N, K, seed=5)
+    q, luts = layer_to_gpu(L)
+    for b in range(3, 9):
+        for M in range(1, 9):
+            print(f"gemv N={N} K={K} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            got = ext.matmul_kbit(xg, q, luts[b], b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+
+
+@pytest.mark.parametrize("N,K", FULL)
+def test_benchmark_shapes(ext, oracle, N, K):
+    L = make(N, K, seed=1)
+    q, luts = layer_to_gpu(L)
+    for b in range(3, 9):
+        for M in (1, 8):
+            print(f"gemv N={N} K={K} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            got = ext.matmul_kbit(xg, q, luts[b], b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+
+
+def test_one_hot_x_returns_dequant_column_exactly(ext, oracle):
+    # with a single 1.0 in x the sum has one non-zero term: the result is the table entry itself
+    N, K = 96, 3104
+    L = make(N, K, seed=8)
+    q, luts = layer_to_gpu(L)
+    for b in (3, 4, 6, 8):
+        w = oracle.dequant_kbit(L.qweight, L.luts[b], b)
+        for k in (0, 7, 8, 255, 256, 1023, 1024, 2047, 2048, 3071, 3072, 3080, 3103):
+            x = torch.zeros((1, K), dtype=torch.float16, device="cuda")
+            x[0, k] = 1.0
+            got = ext.matmul_kbit(x, q, luts[b], b)
+            assert_bit_exact(got[0], w[:, k], f"b={b} k={k}")
+
+
+def test_constant_table_gives_scaled_sum(ext):
+    N, K = 64, 11008
+    L = make(N, K, seed=2)
+    q, _ = layer_to_gpu(L)
+    x, xg = _x(2, K)
+    lut = torch.full((N, 32), 0.5, dtype=torch.float16, device="cuda")
+    got = ext.matmul_kbit(xg, q, lut, 5)
+    want = 0.5 * x.astype(np.float64).sum(axis=1, keepdims=True) * np.ones((1, N))
+    assert_close_gemv(got, want, "constant table")
+
+
+def test_leading_dims_and_determinism(ext, oracle):
+    N, K = 512, 4096
+    L = make(N, K, seed=3)
+    q, luts = layer_to_gpu(L)
+    x = synth.make_x(6, K).reshape(2, 3, K)
+    xg = torch.from_numpy(x).cuda()
+    a = ext.matmul_kbit(xg, q, luts[6], 6)
+    assert a.shape == (2, 3, N)
+    b = ext.matmul_kbit(xg.reshape(6, K), q, luts[6], 6)
+    assert torch.equal(a.reshape(6, N).view(torch.int16), b.view(torch.int16))
+    for _ in range(3):
+        assert torch.equal(ext.matmul_kbit(xg, q, luts[6], 6).view(torch.int16), a.view(torch.int16))
+    v = ext.matmul_kbit(xg[0, 0], q, luts[6], 6)      # 1-D input, as the reference allows
+    assert v.shape == (N,)
+
+
+def test_pruned_planes(ext, oracle):
+    L = make(64, 4096, seed=9)
+    x, xg = _x(1, 4096)
+    for b in range(3, 9):
+        q, luts = layer_to_gpu(L, planes=b)
+        _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+        assert_close_gemv(ext.matmul_kbit(xg, q, luts[b], b), want, f"b={b}")
+
+
+def test_batch_above_8_is_rejected_like_the_reference_assert(ext):
+    L = make(8, 64, seed=0)
+    q, luts = layer_to_gpu(L)
+    with pytest.raises(ValueError, match="1..8"):
+        ext.matmul_kbit(torch.zeros((9, 64), dtype=torch.float16, device="cuda"), q, luts[3], 3)
+    with pytest.raises(ValueError, match="planes"):
+        ext.matmul_kbit(torch.zeros((1, 64), dtype=torch.float16, device="cuda"), q[:3].contiguous(), luts[4], 4)
+    with pytest.raises(ValueError, match="contiguous"):
+        ext.matmul_kbit(torch.zeros((1, 128), dtype=torch.float16, device="cuda")[:, ::2], q, luts[3], 3)
+
+
+def test_graph_replay_matches_eager(ext):
+    from any_precision_amd import _capi
+    N, K = 1024, 4096
+    L = make(N, K, seed=4)
+    q, luts = layer_to_gpu(L)
+    _, xg = _x(1, K)
+    eager = ext.matmul_kbit(xg, q, luts[4], 4)
+    out = torch.zeros((1, N), dtype=torch.float16, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        rc = _capi.lib.ap_matmul_kbit(xg.data_ptr(), q.data_ptr(), luts[4].data_ptr(), out.data_ptr(), 1, N, K, 4,
+                                      torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+    for rep in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), rep

@@ -1,0 +1,83 @@
+"""The kernels' pure-integer helpers (ap_bitplane.hpp), built for the host with
+g++, against the oracle and against the layout definition (CPU only)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+
+def _run(hostcheck, q, bits, shift=0):
+    q = np.ascontiguousarray(q, dtype=np.uint32)
+    out = np.zeros(8, dtype=np.uint32)
+    rc = hostcheck.aph_planes_to_indices(ctypes.c_void_p(q.ctypes.data), bits, shift, ctypes.c_void_p(out.ctypes.data))
+    assert rc == 0
+    return out
+
+
+@pytest.mark.parametrize("bits", range(1, 9))
+def test_butterfly_transpose_matches_oracle(hostcheck, oracle, bits):
+    rng = np.random.default_rng(bits)
+    for _ in range(300):
+        q = rng.integers(0, 2**32, size=bits, dtype=np.uint64).astype(np.uint32)
+        assert np.array_equal(_run(hostcheck, q, bits), oracle.transpose(q, bits))
+    for p in range(bits):                    # walking ones / zeros
+        for pos in range(32):
+            q = np.zeros(bits, dtype=np.uint32)
+            q[p] = np.uint32(1 << pos)
+            assert np.array_equal(_run(hostcheck, q, bits), oracle.transpose(q, bits))
+            q = ~q
+            assert np.array_equal(_run(hostcheck, q, bits), oracle.transpose(q, bits))
+
+
+@pytest.mark.parametrize("bits", range(3, 8))
+def test_preshifted_indices(hostcheck, oracle, bits):
+    rng = np.random.default_rng(40 + bits)
+    for _ in range(100):
+        q = rng.integers(0, 2**32, size=bits, dtype=np.uint64).astype(np.uint32)
+        assert np.array_equal(_run(hostcheck, q, bits, 1), oracle.transpose(q, bits) << np.uint32(1))
+
+
+@pytest.mark.parametrize("bits", [3, 4])
+def test_pair_indices(hostcheck, oracle, bits):
+    rng = np.random.default_rng(50 + bits)
+    for _ in range(200):
+        q = rng.integers(0, 2**32, size=bits, dtype=np.uint64).astype(np.uint32)
+        out = np.zeros(4, dtype=np.uint32)
+        assert hostcheck.aph_planes_to_pair_indices(ctypes.c_void_p(q.ctypes.data), bits,
+                                                    ctypes.c_void_p(out.ctypes.data)) == 0
+        assert np.array_equal(out, oracle.transpose_pair(q, bits))
+
+
+@pytest.mark.parametrize("K", [32, 64, 992, 1024, 1056, 4096, 11008, 14336])
+def test_group_base_enumerates_every_element_once(hostcheck, K):
+    W = K // 32
+    seen = np.zeros(K, dtype=np.int32)
+    for w in range(W):
+        T = hostcheck.aph_chunk_words(w, K)
+        assert T == (32 if (w // 32) < K // 1024 else (K % 1024) // 32)
+        for j in range(4):
+            k0 = hostcheck.aph_group_base(w, j, K)
+            assert k0 % 8 == 0 and 0 <= k0 <= K - 8
+            seen[k0:k0 + 8] += 1
+    assert (seen == 1).all()
+
+
+def test_group_base_matches_packer(hostcheck, oracle):
+    # a one-hot code at element k must show up in word w, byte group j, bit e as the helper says
+    K = 1056 + 64
+    W = K // 32
+    where = {}
+    for w in range(W):
+        for j in range(4):
+            k0 = hostcheck.aph_group_base(w, j, K)
+            for e in range(8):
+                where[k0 + e] = (w, 8 * (3 - j) + 7 - e)
+    rng = np.random.default_rng(1)
+    for k in rng.choice(K, size=80, replace=False):
+        codes = np.zeros((1, K), dtype=np.uint8)
+        codes[0, k] = 0x80
+        qw = oracle.pack_bitplanes(codes, 8).view(np.uint32)[0, 0]
+        w, bit = where[int(k)]
+        expect = np.zeros(W, dtype=np.uint32)
+        expect[w] = np.uint32(1 << bit)
+        assert np.array_equal(qw, expect)
