@@ -70,13 +70,23 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     return AP_OK;
 }
 
+template <int BITS, int M, int WPL, int THREADS>
+void launch_gemv_t(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                   uint16_t *out, int N, int K, hipStream_t stream) {
+    const dim3 block(kWave, geo.S, geo.G);
+    gemv_kbit_kernel<BITS, M, WPL, THREADS><<<dim3(geo.grid), block, 0, stream>>>(
+        reinterpret_cast<const half_t *>(x), qweight, reinterpret_cast<const half_t *>(lut),
+        reinterpret_cast<half_t *>(out), N, K, geo.R);
+}
+
+// Smallest workgroup bound that holds S*G waves: leaves the most registers per lane.
 template <int BITS, int M, int WPL>
 void launch_gemv(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int N, int K, hipStream_t stream) {
-    const dim3 block(kWave, geo.S, geo.G);
-    gemv_kbit_kernel<BITS, M, WPL><<<dim3(geo.grid), block, 0, stream>>>(
-        reinterpret_cast<const half_t *>(x), qweight, reinterpret_cast<const half_t *>(lut),
-        reinterpret_cast<half_t *>(out), N, K, geo.R);
+    const int waves = geo.S * geo.G;
+    if (waves <= 4) return launch_gemv_t<BITS, M, WPL, 256>(geo, x, qweight, lut, out, N, K, stream);
+    if (waves <= 8) return launch_gemv_t<BITS, M, WPL, 512>(geo, x, qweight, lut, out, N, K, stream);
+    launch_gemv_t<BITS, M, WPL, 1024>(geo, x, qweight, lut, out, N, K, stream);
 }
 
 template <int BITS, int M>

@@ -40,16 +40,19 @@ __device__ __forceinline__ uint32_t word_of(const typename WordVec<WPL>::type &v
 }
 
 // Grid: ceil(N / (G*R)) workgroups of (64, S, G) threads.  Host guarantees
-// W % WPL == 0, S*G <= kGemvMaxWaves, R <= kGemvMaxRows, S*64*WPL >= W.
-template <int BITS, int M, int WPL>
-__global__ __launch_bounds__(kGemvMaxWaves * kWave) void gemv_kbit_kernel(
+// W % WPL == 0, S*G*64 <= THREADS, R <= kGemvMaxRows, S*64*WPL >= W.
+// THREADS (256, 512 or 1024) only bounds the workgroup size so that small
+// workgroups may use more registers per lane (M x WPL x 16 of them hold x).
+template <int BITS, int M, int WPL, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
     const half_t *__restrict__ lut, half_t *__restrict__ out,
     int N, int K, int R) {
     constexpr int NC = 1 << BITS;
     typedef typename WordVec<WPL>::type wvec_t;
-    __shared__ __attribute__((aligned(16))) half_t tables[kGemvMaxWaves][2][NC];
-    __shared__ float partial[kGemvMaxWaves * kGemvMaxRows * M];
+    constexpr int MAXW = THREADS / kWave;
+    __shared__ __attribute__((aligned(16))) half_t tables[MAXW][2][NC];
+    __shared__ float partial[MAXW * kGemvMaxRows * M];
 
     const int lane = threadIdx.x;
     const int s = threadIdx.y, S = blockDim.y;

@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the bitplane GEMV (matmul_kbit) on one MI355X.
+
+Workload (the configuration the headline metric is quoted on): the seven linears of one
+Llama-2-7B decoder layer at batch 1 -- q,k,v,o 4096x4096, gate,up 11008x4096, down
+4096x11008 -- parent 8 bits, every w_bits in 3..8.  One "step" is one pass over those
+7 x 6 = 42 GEMVs.  Weights live in HBM before the timed region; consecutive steps walk a
+pool of distinct layers so that no launch finds its planes in the 256 MB last-level cache.
+
+Prints ONE JSON line: whole-step effective bandwidth (algorithmic bytes / time), the
+per-kernel roofline of the kernel that dominates the step, and the CPU baseline (the C
+oracle's host-speed GEMV on the same shapes, timed on this box's cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "any-precision-llm_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+BITS = (3, 4, 5, 6, 7, 8)
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--pool", type=int, default=4, help="distinct decoder layers the steps rotate over")
+    ap.add_argument("--kernel-reps", type=int, default=40, help="launches per (shape, w_bits) for the per-kernel table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--table", default="", help="also write the per-layer table (markdown) to this file")
+    ap.add_argument("--only-step", action="store_true", help="skip the per-kernel table (used under rocprofv3)")
+    return ap.parse_args()
+
+
+class Layer:
+    """Device-resident synthetic linear: uniform parent codes are uniform plane bits, so the
+    planes are drawn directly as random words; tables are ascending N(0, 0.02) draws."""
+
+    def __init__(self, torch, N, K, gen):
+        self.N, self.K = N, K
+        self.qweight = torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda",
+                                     generator=gen)
+        self.luts = {}
+        for b in BITS:
+            t = torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02
+            self.luts[b] = torch.sort(t, dim=1).values.to(torch.float16).contiguous()
+        self.out = torch.empty((1, N), dtype=torch.float16, device="cuda")
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from any_precision_amd import _capi, synth
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    shapes = [(n, N, K) for n, N, K in synth.LLAMA2_7B_LAYER]
+
+    pool = [[Layer(torch, N, K, gen) for _, N, K in shapes] for _ in range(args.pool)]
+    xs = {K: torch.randn((1, K), device="cuda", generator=gen).to(torch.float16) for K in {K for _, _, K in shapes}}
+    torch.cuda.synchronize()
+
+    def launch(layer: Layer, b: int, stream: int):
+        rc = lib.ap_matmul_kbit(xs[layer.K].data_ptr(), layer.qweight.data_ptr(), layer.luts[b].data_ptr(),
+                                layer.out.data_ptr(), 1, layer.N, layer.K, b, stream)
+        if rc != 0:
+            raise RuntimeError(_capi.strerror(rc))
+
+    def step(i: int, stream: int):
+        for b in BITS:
+            for layer in pool[i % args.pool]:
+                launch(layer, b, stream)
+
+    step_bytes = sum(synth.gemv_bytes(N, K, b, 1) for _, N, K in shapes for b in BITS)
+
+    # ---- whole-step timing: the K steps are captured in one HIP graph so the host never starves the GPU
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(args.warmup):
+            step(i, side.cuda_stream)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(args.steps):
+                step(args.warmup + i, torch.cuda.current_stream().cuda_stream)
+        graph.replay()                      # untimed: first replay pays graph upload
+        side.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(side)
+        graph.replay()
+        e1.record(side)
+        torch.cuda.synchronize()
+        total_ms = e0.elapsed_time(e1)
+    ms_per_step = total_ms / args.steps
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-kernel table: each (shape, w_bits) alone, rotating over the pool (cold planes)
+    table = []
+    if not args.only_step:
+        uniq = {}
+        for idx, (name, N, K) in enumerate(shapes):
+            uniq.setdefault((N, K), []).append(idx)
+        with torch.cuda.stream(side):
+            for (N, K), idxs in uniq.items():
+                layers = [pool[p][i] for p in range(args.pool) for i in idxs]
+                for b in BITS:
+                    g = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(g, stream=side):
+                        for r in range(args.kernel_reps):
+                            launch(layers[r % len(layers)], b, torch.cuda.current_stream().cuda_stream)
+                    g.replay()
+                    side.synchronize()
+                    a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a0.record(side)
+                    g.replay()
+                    a1.record(side)
+                    side.synchronize()
+                    us = a0.elapsed_time(a1) * 1e3 / args.kernel_reps
+                    by = synth.gemv_bytes(N, K, b, 1)
+                    geo = _capi.matmul_geometry(1, N, K, b)
+                    table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 3), "GBps": round(by / us / 1e3, 1),
+                                  "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": by,
+                                  "count_in_step": len(idxs), "geometry": geo})
+
+    roofline = None
+    if table:
+        dom = max(table, key=lambda r: r["us"] * r["count_in_step"])
+        roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": dom["frac"], "traffic": None,
+                    "kernel": f"gemv_kbit_kernel<{dom['w_bits']},1,{dom['geometry']['wpl']},*> {dom['N']}x{dom['K']}",
+                    "us_per_launch": dom["us"], "algorithmic_bytes_per_launch": dom["bytes"]}
+
+    # ---- CPU baseline: the oracle's host-speed GEMV (unpack + gather + dot), same shapes
+    cpu = None
+    if not args.no_cpu:
+        import numpy as np
+        import oracle
+        oracle.build()
+        rng = np.random.default_rng(0)
+        cpu_bits = (3, 8)
+        t_cpu, b_cpu = 0.0, 0
+        for _, N, K in [shapes[0], shapes[4], shapes[6]]:
+            qw = rng.integers(-2**31, 2**31 - 1, size=(8, N, K // 32), dtype=np.int64).astype(np.int32)
+            x = rng.normal(0, 1, size=(1, K)).astype(np.float16)
+            for b in cpu_bits:
+                lut = np.sort(rng.normal(0, 0.02, size=(N, 1 << b)), axis=1).astype(np.float16)
+                oracle.matmul_kbit_fast(x, qw, lut, b)                  # warm
+                reps = 3
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    oracle.matmul_kbit_fast(x, qw, lut, b)
+                t_cpu += (time.perf_counter() - t0) / reps
+                b_cpu += synth.gemv_bytes(N, K, b, 1)
+        cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+               "sample": "C oracle GEMV (unpack+gather+fp32 dot, OpenMP over rows): 4096x4096, 11008x4096, "
+                         "4096x11008 at w_bits 3 and 8, batch 1, mean of 3 runs each"}
+
+    result = {
+        "metric": "bitplane GEMV effective HBM GB/s, Llama-2-7B layer set, w_bits 3-8, batch 1",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "Llama-2-7B decoder-layer linear set (q,k,v,o 4096x4096; gate,up 11008x4096; "
+                               "down 4096x11008), batch 1, parent 8 bits, w_bits 3..8 = 42 GEMVs per step",
+                   "pool_layers": args.pool, "bytes_per_step": step_bytes,
+                   "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
+        "roofline": roofline, "cpu_baseline": cpu, "layers": table,
+    }
+    if args.table and table:
+        with open(args.table, "w") as f:
+            f.write("| N x K | w_bits | us/launch | GB/s | % of 8 TB/s |\n|---|---|---|---|---|\n")
+            for r in table:
+                f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | {r['us']:.2f} | {r['GBps']:.0f} | {100 * r['frac']:.1f} |\n")
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
