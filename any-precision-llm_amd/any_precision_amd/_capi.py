@@ -32,7 +32,7 @@ lib.ap_dequant_kbit.restype = _ci
 lib.ap_matmul_kbit.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 lib.ap_matmul_kbit.restype = _ci
 _pi = ctypes.POINTER(ctypes.c_int)
-lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi, _pi]
+lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi]
 lib.ap_matmul_kbit_geometry.restype = _ci
 
 if lib.ap_abi_version() != AP_ABI_VERSION:
@@ -57,6 +57,6 @@ def check(code: int, what: str) -> None:
 
 
 def matmul_geometry(M: int, N: int, K: int, w_bits: int) -> dict:
-    vals = [ctypes.c_int() for _ in range(5)]
+    vals = [ctypes.c_int() for _ in range(4)]
     check(lib.ap_matmul_kbit_geometry(M, N, K, w_bits, *[ctypes.byref(v) for v in vals]), "ap_matmul_kbit_geometry")
-    return dict(zip(("wpl", "segments", "groups", "rows", "grid"), (v.value for v in vals)))
+    return dict(zip(("wpl", "segments", "rows", "grid"), (v.value for v in vals)))

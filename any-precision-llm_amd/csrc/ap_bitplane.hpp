@@ -32,13 +32,36 @@ AP_HD int group_base(int w, int j, int K) {
     return (c << 10) + 8 * (chunk_words(w, K) * j + t);
 }
 
-// One butterfly step of an 8x8 bit-matrix transpose carried out in the four
-// byte columns of a word at once: exchanges the S-bit blocks selected by
-// `lo_mask` between word a (keeps its low blocks) and word b (keeps its high).
-template <int S, uint32_t LO>
+// (a & mask) | (b & ~mask): one v_bitop3_b32 on the GPU.
+AP_HD uint32_t bit_select(uint32_t mask, uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_bitop3_b32(a, b, mask, 0xE4);
+#else
+    return (a & mask) | (b & ~mask);
+#endif
+}
+
+// One butterfly step of a bit-matrix transpose carried out in every byte (or
+// nibble) of a word at once: exchanges the S-bit blocks selected by LO
+// between word a (keeps its low blocks) and word b (keeps its high blocks).
+// Each output is one shift and one three-input bitwise select; AZERO / BZERO
+// say that a / b is known to be zero, which saves the select.
+template <int S, uint32_t LO, bool AZERO = false, bool BZERO = false>
 AP_HD void swap_blocks(uint32_t &a, uint32_t &b) {
-    const uint32_t na = (a & LO) | ((b << S) & ~LO);
-    const uint32_t nb = ((a >> S) & LO) | (b & ~LO);
+    uint32_t na, nb;
+    if constexpr (AZERO && BZERO) {
+        na = 0u;
+        nb = 0u;
+    } else if constexpr (BZERO) {
+        na = a & LO;
+        nb = (a >> S) & LO;
+    } else if constexpr (AZERO) {
+        na = (b << S) & ~LO;
+        nb = b & ~LO;
+    } else {
+        na = bit_select(LO, a, b << S);
+        nb = bit_select(LO, a >> S, b);
+    }
     a = na;
     b = nb;
 }
@@ -52,36 +75,83 @@ AP_HD void swap_blocks(uint32_t &a, uint32_t &b) {
 template <int BITS, int SHIFT = 0>
 AP_HD void planes_to_indices(const uint32_t (&q)[BITS], uint32_t (&idx)[8]) {
     static_assert(BITS >= 1 && BITS + SHIFT <= 8, "index must fit a byte");
+    // row i feeds bit i of the output byte: plane BITS-1-(i-SHIFT), zero outside
+    constexpr int LOW = SHIFT, HIGH = SHIFT + BITS;   // rows [LOW, HIGH) are live
+#define AP_LIVE(i) ((i) >= LOW && (i) < HIGH)
     uint32_t r[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        // bit i of the output byte comes from row i: plane BITS-1-(i-SHIFT)
-        const int p = BITS - 1 - (i - SHIFT);
-        r[i] = (p >= 0 && p < BITS) ? q[p >= 0 && p < BITS ? p : 0] : 0u;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++) swap_blocks<4, 0x0F0F0F0Fu>(r[i], r[i + 4]);
-#pragma unroll
-    for (int i = 0; i < 8; i += 4) {
-        swap_blocks<2, 0x33333333u>(r[i], r[i + 2]);
-        swap_blocks<2, 0x33333333u>(r[i + 1], r[i + 3]);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; i += 2) swap_blocks<1, 0x55555555u>(r[i], r[i + 1]);
+    for (int i = 0; i < 8; i++) r[i] = AP_LIVE(i) ? q[AP_LIVE(i) ? BITS - 1 - (i - SHIFT) : 0] : 0u;
+    // stage 1: 4-bit blocks between rows i and i+4
+    swap_blocks<4, 0x0F0F0F0Fu, !AP_LIVE(0), !AP_LIVE(4)>(r[0], r[4]);
+    swap_blocks<4, 0x0F0F0F0Fu, !AP_LIVE(1), !AP_LIVE(5)>(r[1], r[5]);
+    swap_blocks<4, 0x0F0F0F0Fu, !AP_LIVE(2), !AP_LIVE(6)>(r[2], r[6]);
+    swap_blocks<4, 0x0F0F0F0Fu, !AP_LIVE(3), !AP_LIVE(7)>(r[3], r[7]);
+    // after stage 1 rows i and i+4 are live iff either was
+#define AP_LIVE1(i) (AP_LIVE((i) & 3) || AP_LIVE(((i) & 3) + 4))
+    swap_blocks<2, 0x33333333u, !AP_LIVE1(0), !AP_LIVE1(2)>(r[0], r[2]);
+    swap_blocks<2, 0x33333333u, !AP_LIVE1(1), !AP_LIVE1(3)>(r[1], r[3]);
+    swap_blocks<2, 0x33333333u, !AP_LIVE1(4), !AP_LIVE1(6)>(r[4], r[6]);
+    swap_blocks<2, 0x33333333u, !AP_LIVE1(5), !AP_LIVE1(7)>(r[5], r[7]);
+#define AP_LIVE2(i) (AP_LIVE1((i) & 5) || AP_LIVE1(((i) & 5) + 2))
+    swap_blocks<1, 0x55555555u, !AP_LIVE2(0), !AP_LIVE2(1)>(r[0], r[1]);
+    swap_blocks<1, 0x55555555u, !AP_LIVE2(2), !AP_LIVE2(3)>(r[2], r[3]);
+    swap_blocks<1, 0x55555555u, !AP_LIVE2(4), !AP_LIVE2(5)>(r[4], r[5]);
+    swap_blocks<1, 0x55555555u, !AP_LIVE2(6), !AP_LIVE2(7)>(r[6], r[7]);
+#undef AP_LIVE2
+#undef AP_LIVE1
+#undef AP_LIVE
     // r[u] byte b bit i = row i bit (8 b + u); element e sits at u = 7 - e.
 #pragma unroll
     for (int e = 0; e < 8; e++) idx[e] = r[7 - e];
 }
 
-// Pair form (reference: dequant<3,true>, dequant<4,true>, dequant.cuh:13-30,
-// 56-67): byte b of pidx[m], m = 0..3, is (index(e = m) << BITS) | index(e = m + 4).
+// Nibble form for BITS <= 4: nib[m], m = 0..3; the high nibble of byte b of
+// nib[m] is the index of element e = m, the low nibble that of e = m + 4, each
+// left-aligned in its nibble (index << (4 - BITS)).  Two butterfly stages.
 template <int BITS>
-AP_HD void planes_to_pair_indices(const uint32_t (&q)[BITS], uint32_t (&pidx)[4]) {
-    static_assert(BITS <= 4, "pair index must fit a byte");
-    uint32_t idx[8];
-    planes_to_indices<BITS, 0>(q, idx);
+AP_HD void planes_to_nibbles(const uint32_t (&q)[BITS], uint32_t (&nib)[4]) {
+    static_assert(BITS >= 1 && BITS <= 4, "index must fit a nibble");
+    // nibble bit i <- plane 3 - i; rows below 4 - BITS are zero
+    constexpr int LOW = 4 - BITS;
+    uint32_t r[4];
 #pragma unroll
-    for (int m = 0; m < 4; m++) pidx[m] = (idx[m] << BITS) | idx[m + 4];
+    for (int i = 0; i < 4; i++) r[i] = (i >= LOW) ? q[i >= LOW ? 3 - i : 0] : 0u;
+    swap_blocks<2, 0x33333333u, (0 < LOW), (2 < LOW)>(r[0], r[2]);
+    swap_blocks<2, 0x33333333u, (1 < LOW), (3 < LOW)>(r[1], r[3]);
+    constexpr bool Z02 = (0 < LOW) && (2 < LOW), Z13 = (1 < LOW) && (3 < LOW);
+    swap_blocks<1, 0x55555555u, Z02, Z13>(r[0], r[1]);
+    swap_blocks<1, 0x55555555u, Z02, Z13>(r[2], r[3]);
+    // r[u] nibble bit i = row i bit u of the nibble; element m sits at u = 3 - m.
+#pragma unroll
+    for (int m = 0; m < 4; m++) nib[m] = r[3 - m];
+}
+
+// Pair form (reference: dequant<3,true>, dequant<4,true>, dequant.cuh:13-30,
+// 56-67): byte b of pidx[m], m = 0..3, is
+//     ((index(e = m) << BITS) | index(e = m + 4)) << SHIFT.
+// BITS = 4, SHIFT = 0: the nibble form itself.  BITS = 3, SHIFT = 1: the high
+// nibble is built right-aligned and the low nibble left-aligned, so the two
+// 3-bit indices come out adjacent -- each butterfly row takes its low nibbles
+// from one plane and its high nibbles from the next.
+template <int BITS, int SHIFT>
+AP_HD void planes_to_pair_indices(const uint32_t (&q)[BITS], uint32_t (&pidx)[4]) {
+    static_assert((BITS == 4 && SHIFT == 0) || (BITS == 3 && SHIFT == 1), "supported pair forms");
+    if constexpr (BITS == 4) {
+        planes_to_nibbles<4>(q, pidx);
+    } else {
+        constexpr uint32_t LO = 0x0F0F0F0Fu;
+        uint32_t r[4];
+        r[3] = q[0] & LO;                    // low nibble bit 3 <- plane 0; high nibble bit 3 stays 0
+        r[2] = bit_select(LO, q[1], q[0]);   // low: plane 1, high: plane 0
+        r[1] = bit_select(LO, q[2], q[1]);   // low: plane 2, high: plane 1
+        r[0] = q[2] & ~LO;                   // low nibble bit 0 stays 0; high: plane 2
+        swap_blocks<2, 0x33333333u>(r[0], r[2]);
+        swap_blocks<2, 0x33333333u>(r[1], r[3]);
+        swap_blocks<1, 0x55555555u>(r[0], r[1]);
+        swap_blocks<1, 0x55555555u>(r[2], r[3]);
+#pragma unroll
+        for (int m = 0; m < 4; m++) pidx[m] = r[3 - m];
+    }
 }
 
 }  // namespace ap

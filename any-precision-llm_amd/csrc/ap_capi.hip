@@ -27,7 +27,7 @@ int env_int(const char *name, int dflt) {
 
 const Tuning &tuning() {
     static const Tuning t = {
-        env_int("AP_GEMV_TARGET_WAVES", 4096),
+        env_int("AP_GEMV_TARGET_WAVES", 16384),
         env_int("AP_GEMV_ROWS", 0),
         env_int("AP_GEMV_WPL", 0),
         env_int("AP_DEQUANT_BLOCKS_PER_CU", 8),
@@ -44,7 +44,8 @@ int check_common(int N, int K, int w_bits) {
 }
 
 struct GemvGeometry {
-    int wpl, S, G, R, grid;
+    int wpl, S, R, G, grid;
+    bool flat;  // everything-prefetched kernel (M <= 2), R in {1, 2, 4}
 };
 
 int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
@@ -57,35 +58,56 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     if (t.force_wpl == 1 || (t.force_wpl == 2 && (W & 1) == 0 && M <= 2)) wpl = t.force_wpl;
     const int seg = kWave * wpl;
     const int S = (W + seg - 1) / seg;
-    if (S > kGemvMaxWaves) return AP_ELIMIT;
-    const int G = S >= 4 ? 1 : (S == 3 ? 1 : 4 / S);
+    if (S > kGemvMaxSeg) return AP_ELIMIT;
     int R = t.force_rows > 0 ? t.force_rows : (int)(((long long)N * S + t.target_waves - 1) / t.target_waves);
     if (R < 1) R = 1;
-    if (R > kGemvMaxRows) R = kGemvMaxRows;
+    geo->flat = (M <= 2);
+    if (geo->flat) {
+        R = R >= 4 ? 4 : (R >= 2 ? 2 : 1);
+    } else if (R > kGemvMaxRows) {
+        R = kGemvMaxRows;
+    }
+    // row groups per workgroup (packing several measured no faster than one)
+    geo->G = 1;
     geo->wpl = wpl;
     geo->S = S;
-    geo->G = G;
     geo->R = R;
-    geo->grid = (N + G * R - 1) / (G * R);
+    geo->grid = (N + R * geo->G - 1) / (R * geo->G);
     return AP_OK;
+}
+
+template <int BITS, int M, int WPL, int R, int THREADS>
+void launch_flat_g(const GemvGeometry &geo, const half_t *x, const uint32_t *qweight, const half_t *lut,
+                   half_t *out, int N, int K, hipStream_t stream) {
+    const dim3 block(kWave, geo.S, geo.G), grid(geo.grid);
+    gemv_kbit_flat_kernel<BITS, M, WPL, R, 1, THREADS><<<grid, block, 0, stream>>>(x, qweight, lut, out, N, K);
 }
 
 template <int BITS, int M, int WPL, int THREADS>
 void launch_gemv_t(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                    uint16_t *out, int N, int K, hipStream_t stream) {
-    const dim3 block(kWave, geo.S, geo.G);
-    gemv_kbit_kernel<BITS, M, WPL, THREADS><<<dim3(geo.grid), block, 0, stream>>>(
-        reinterpret_cast<const half_t *>(x), qweight, reinterpret_cast<const half_t *>(lut),
-        reinterpret_cast<half_t *>(out), N, K, geo.R);
+    const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
+    half_t *oh = reinterpret_cast<half_t *>(out);
+    if constexpr (M <= 2 && THREADS != 512) {
+        switch (geo.R) {
+            case 1: return launch_flat_g<BITS, M, WPL, 1, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
+            case 2: return launch_flat_g<BITS, M, WPL, 2, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
+            default: return launch_flat_g<BITS, M, WPL, 4, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
+        }
+    } else if constexpr (M > 2) {
+        const dim3 block(kWave, geo.S), grid(geo.grid);
+        gemv_kbit_kernel<BITS, M, WPL, THREADS><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, N, K, geo.R);
+    }
 }
 
-// Smallest workgroup bound that holds S*G waves: leaves the most registers per lane.
+// Smallest workgroup bound that holds S waves: leaves the most registers per lane.
 template <int BITS, int M, int WPL>
 void launch_gemv(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int N, int K, hipStream_t stream) {
-    const int waves = geo.S * geo.G;
-    if (waves <= 4) return launch_gemv_t<BITS, M, WPL, 256>(geo, x, qweight, lut, out, N, K, stream);
-    if (waves <= 8) return launch_gemv_t<BITS, M, WPL, 512>(geo, x, qweight, lut, out, N, K, stream);
+    if (geo.S <= 4) return launch_gemv_t<BITS, M, WPL, 256>(geo, x, qweight, lut, out, N, K, stream);
+    if constexpr (M > 2) {
+        if (geo.S <= 8) return launch_gemv_t<BITS, M, WPL, 512>(geo, x, qweight, lut, out, N, K, stream);
+    }
     launch_gemv_t<BITS, M, WPL, 1024>(geo, x, qweight, lut, out, N, K, stream);
 }
 
@@ -166,14 +188,12 @@ int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
     return launch_status();
 }
 
-int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segments, int *groups, int *rows,
-                            int *grid) {
+int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segments, int *rows, int *grid) {
     GemvGeometry geo;
     const int rc = gemv_geometry(M, N, K, w_bits, &geo);
     if (rc != AP_OK) return rc;
     if (wpl) *wpl = geo.wpl;
     if (segments) *segments = geo.S;
-    if (groups) *groups = geo.G;
     if (rows) *rows = geo.R;
     if (grid) *grid = geo.grid;
     return AP_OK;

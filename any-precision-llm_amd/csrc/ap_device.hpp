@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace ap {
 
 typedef _Float16 half_t;
@@ -13,9 +15,45 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWave = 64;
 
+// Compile-time loop: f(integral_constant<int,0>) ... f(integral_constant<int,N-1>).
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
 // fp32 += a.x*b.x + a.y*b.y  (v_dot2c_f32_f16: fp16 products, fp32 accumulate)
 __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
     return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, w), __builtin_bit_cast(half2_t, x), acc, false);
+}
+
+// ((v >> 8*BYTE) & 0xff) << SHIFT in one VALU instruction: SDWA byte select on
+// the shifted operand (SHIFT > 0), a bit-field extract otherwise.  This is the
+// LDS byte offset of a gather whose table sits at a compile-time address.
+template <int BYTE, int SHIFT>
+__device__ __forceinline__ uint32_t byte_offset(uint32_t v) {
+    static_assert(BYTE >= 0 && BYTE < 4 && SHIFT >= 0 && SHIFT < 8, "");
+    if constexpr (SHIFT == 0) {
+        return __builtin_amdgcn_ubfe(v, 8 * BYTE, 8);
+    } else {
+        uint32_t r;
+        const uint32_t sh = SHIFT;
+        if constexpr (BYTE == 0)
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
+                : "=v"(r) : "v"(sh), "v"(v));
+        else if constexpr (BYTE == 1)
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1"
+                : "=v"(r) : "v"(sh), "v"(v));
+        else if constexpr (BYTE == 2)
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2"
+                : "=v"(r) : "v"(sh), "v"(v));
+        else
+            asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3"
+                : "=v"(r) : "v"(sh), "v"(v));
+        return r;
+    }
 }
 
 template <int CTRL>

@@ -5,25 +5,44 @@
 // (any_precision/modules/kernels/matmul.cuh:16-167); the reference sums in
 // fp16, this kernel in fp32.
 //
-// Mapping (wave64): a workgroup is S x G waves.  Wave (s,g) owns K-segment s
-// (64*WPL consecutive words of a row = 2048*WPL elements) of the rows of row
-// group g.  The activations a lane needs never change from row to row, so
-// they are loaded once into registers, already ordered the way the packed
-// layout scatters elements (4 runs of 8 consecutive elements per word).  Per
-// row a lane then streams WPL words per plane (one 4*WPL-byte load per plane,
-// a wave covers 256*WPL contiguous bytes), rebuilds its indices in registers,
-// gathers from the row's table in this wave's LDS slot and feeds
-// v_dot2c_f32_f16.  Lane partials are summed with DPP; when S > 1 the S
-// segment partials of a row meet in LDS and are added in a fixed order, so the
-// result is deterministic.
+// The kernel is bound by VALU and LDS-gather issue rather than by HBM at low
+// bit-widths (a table lookup per weight), so the design minimises instructions
+// per weight:
+//   * A workgroup is S waves that walk the same R consecutive rows together;
+//     wave s owns K-segment s (64*WPL consecutive words = 2048*WPL elements).
+//     One row is in flight per workgroup, so the row's table sits at a
+//     compile-time LDS address and a gather address is a single SDWA
+//     byte-extract-and-shift.
+//   * The activations a lane needs are the same for every row: they are loaded
+//     once into registers, already permuted into the order the packed layout
+//     scatters elements.
+//   * Per row a lane streams WPL words per plane (one load per plane, a wave
+//     covers 256*WPL contiguous bytes), rebuilds its indices with a butterfly
+//     transpose in registers, gathers from LDS and feeds v_dot2c_f32_f16.
+//   * 3 and 4 bits use a pair table (reference idea: matmul.cuh:24,41-49,
+//     dequant.cuh:13-30,56-67): 4^b entries of two fp16 (w[e], w[e+4]), one
+//     32-bit gather per two weights and no packing.  5..8 bits gather single
+//     fp16 entries and pack two of them per dot2.
+//   * Next row's planes and table are prefetched while the current row is
+//     computed; tables are double-buffered so one barrier per row suffices.
+//   * Lane partials are summed with DPP; when S > 1 the segment partials of a
+//     row meet in LDS and are added in a fixed order: results are deterministic.
 #pragma once
+#include <type_traits>
+
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
 
 namespace ap {
 
-constexpr int kGemvMaxWaves = 16;  // S * G upper bound (1024 threads)
-constexpr int kGemvMaxRows = 8;    // rows per wave upper bound (R)
+constexpr int kGemvMaxSeg = 16;   // K-segments (waves) per workgroup
+constexpr int kGemvMaxRows = 16;  // rows per workgroup upper bound (R)
+
+template <int BITS>
+struct GemvTable {
+    static constexpr bool kPair = BITS <= 4;
+    static constexpr int kBytes = kPair ? (4 << (2 * BITS)) : (2 << BITS);
+};
 
 template <int WPL>
 struct WordVec;
@@ -31,42 +50,77 @@ template <>
 struct WordVec<1> { typedef uint32_t type; };
 template <>
 struct WordVec<2> { typedef u32x2 type; };
-template <>
-struct WordVec<4> { typedef u32x4 type; };
 
 template <int WPL>
 __device__ __forceinline__ uint32_t word_of(const typename WordVec<WPL>::type &v, int i) {
     if constexpr (WPL == 1) return v; else return v[i];
 }
 
-// Grid: ceil(N / (G*R)) workgroups of (64, S, G) threads.  Host guarantees
-// W % WPL == 0, S*G*64 <= THREADS, R <= kGemvMaxRows, S*64*WPL >= W.
-// THREADS (256, 512 or 1024) only bounds the workgroup size so that small
-// workgroups may use more registers per lane (M x WPL x 16 of them hold x).
-template <int BITS, int M, int WPL, int THREADS>
-__global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
-    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
-    const half_t *__restrict__ lut, half_t *__restrict__ out,
-    int N, int K, int R) {
-    constexpr int NC = 1 << BITS;
-    typedef typename WordVec<WPL>::type wvec_t;
-    constexpr int MAXW = THREADS / kWave;
-    __shared__ __attribute__((aligned(16))) half_t tables[MAXW][2][NC];
-    __shared__ float partial[MAXW * kGemvMaxRows * M];
+// Registers that carry one row's table from global memory to LDS.
+template <int BITS>
+struct TableRegs {
+    uint32_t a;
+    u32x2 b;
+};
 
-    const int lane = threadIdx.x;
-    const int s = threadIdx.y, S = blockDim.y;
-    const int g = threadIdx.z, G = blockDim.z;
-    const int wave = g * S + s;
-    const int W = K >> 5;
-    const size_t plane_stride = (size_t)N * W;
+// Issue the global loads of row `lut_row` (2^BITS fp16) for this lane.
+template <int BITS>
+__device__ __forceinline__ TableRegs<BITS> table_fetch(const half_t *lut_row, int lane) {
+    TableRegs<BITS> r;
+    r.a = 0u;
+    r.b = u32x2{0u, 0u};
+    const uint16_t *l16 = reinterpret_cast<const uint16_t *>(lut_row);
+    if constexpr (BITS == 3) {          // entry `lane` = (lut[lane >> 3], lut[lane & 7])
+        r.a = l16[lane >> 3];
+        r.b.x = l16[lane & 7];
+    } else if constexpr (BITS == 4) {   // entries 4*lane .. 4*lane+3 = (lut[lane >> 2], lut[4*(lane&3) + i])
+        r.a = l16[lane >> 2];
+        r.b = reinterpret_cast<const u32x2 *>(lut_row)[lane & 3];
+    } else if constexpr (BITS == 8) {   // 512 B: 64 lanes x 8 B
+        r.b = reinterpret_cast<const u32x2 *>(lut_row)[lane];
+    } else if constexpr (BITS == 7) {   // 256 B: 64 lanes x 4 B
+        r.a = reinterpret_cast<const uint32_t *>(lut_row)[lane];
+    } else {                            // 64 / 128 B: first lanes x 4 B
+        if (lane < (1 << BITS) / 2) r.a = reinterpret_cast<const uint32_t *>(lut_row)[lane];
+    }
+    return r;
+}
 
-    const int w0 = (s * kWave + lane) * WPL;
-    const bool valid = w0 < W;
-    const int wl = valid ? w0 : 0;  // inactive lanes read word 0 and are zeroed below
+// Write the fetched table into LDS in the form the gathers expect.
+template <int BITS>
+__device__ __forceinline__ void table_stage(const TableRegs<BITS> &r, uint8_t *slot, int lane) {
+    if constexpr (BITS == 3) {
+        reinterpret_cast<uint32_t *>(slot)[lane] = r.a | (r.b.x << 16);
+    } else if constexpr (BITS == 4) {
+        u32x4 v;
+        v[0] = r.a | (r.b.x << 16);
+        v[1] = r.a | (r.b.x & 0xffff0000u);
+        v[2] = r.a | (r.b.y << 16);
+        v[3] = r.a | (r.b.y & 0xffff0000u);
+        reinterpret_cast<u32x4 *>(slot)[lane] = v;
+    } else if constexpr (BITS == 8) {
+        reinterpret_cast<u32x2 *>(slot)[lane] = r.b;
+    } else if constexpr (BITS == 7) {
+        reinterpret_cast<uint32_t *>(slot)[lane] = r.a;
+    } else {
+        if (lane < (1 << BITS) / 2) reinterpret_cast<uint32_t *>(slot)[lane] = r.a;
+    }
+}
 
-    // Activations for this lane's words, in packed-layout order.
-    u32x4 X[M][WPL][4];
+// Workgroup barrier that orders LDS traffic only: outstanding global loads
+// (the prefetch of the next row) stay in flight across it.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Activations of one lane's words, loaded once per wave.  X[m][wi][j][i] multiplies
+// the weight pair gathered for byte group j of word wi: elements (2i, 2i+1) of the
+// group, or (i, i+4) in pair-table mode.
+template <int BITS, int M, int WPL>
+__device__ __forceinline__ void load_activations(const half_t *__restrict__ x, int K, int wl,
+                                                 uint32_t (&X)[M][WPL][4][4]) {
 #pragma unroll
     for (int m = 0; m < M; m++)
 #pragma unroll
@@ -74,87 +128,237 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + group_base(wl + wi, j, K));
-                X[m][wi][j] = valid ? v : u32x4{0u, 0u, 0u, 0u};
+                if constexpr (GemvTable<BITS>::kPair) {
+                    X[m][wi][j][0] = __builtin_amdgcn_perm(v[2], v[0], 0x05040100u);
+                    X[m][wi][j][1] = __builtin_amdgcn_perm(v[2], v[0], 0x07060302u);
+                    X[m][wi][j][2] = __builtin_amdgcn_perm(v[3], v[1], 0x05040100u);
+                    X[m][wi][j][3] = __builtin_amdgcn_perm(v[3], v[1], 0x07060302u);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) X[m][wi][j][i] = v[i];
+                }
             }
+}
 
-    const int row0 = blockIdx.x * (G * R) + g;
-    half_t(*tab)[NC] = tables[wave];
+// One row x one lane: rebuild the indices of this lane's WPL words, gather from
+// `table` (an LDS array at a compile-time address) and accumulate the M dot products.
+template <int BITS, int M, int WPL>
+__device__ __forceinline__ void row_dot(const typename WordVec<WPL>::type (&q)[BITS],
+                                        const uint8_t (&table)[GemvTable<BITS>::kBytes],
+                                        const uint32_t (&X)[M][WPL][4][4], float (&acc)[M][2]) {
+#pragma unroll
+    for (int wi = 0; wi < WPL; wi++) {
+        uint32_t qq[BITS];
+#pragma unroll
+        for (int p = 0; p < BITS; p++) qq[p] = word_of<WPL>(q[p], wi);
+        if constexpr (GemvTable<BITS>::kPair) {
+            uint32_t pidx[4];
+            // byte = pair index (4 bits) or pair index << 1 (3 bits); a table entry is 4 bytes
+            planes_to_pair_indices<BITS, BITS == 3 ? 1 : 0>(qq, pidx);
+            auto gather_pair = [&](auto i_c, auto c_c) {
+                constexpr int i = decltype(i_c)::value, c = decltype(c_c)::value;
+                const uint32_t off = byte_offset<c, BITS == 4 ? 2 : 1>(pidx[i]);
+                const uint32_t w2 = *reinterpret_cast<const uint32_t *>(&table[off]);
+#pragma unroll
+                for (int m = 0; m < M; m++) acc[m][c & 1] = dot2(w2, X[m][wi][3 - c][i], acc[m][c & 1]);
+            };
+            static_for<4>([&](auto i_c) { static_for<4>([&](auto c_c) { gather_pair(i_c, c_c); }); });
+        } else {
+            uint32_t idx[8];
+            planes_to_indices<BITS>(qq, idx);
+            auto gather_two = [&](auto i_c, auto c_c) {
+                constexpr int i = decltype(i_c)::value, c = decltype(c_c)::value;
+                const uint32_t o0 = byte_offset<c, 1>(idx[2 * i]);
+                const uint32_t o1 = byte_offset<c, 1>(idx[2 * i + 1]);
+                const uint32_t lo = *reinterpret_cast<const uint16_t *>(&table[o0]);
+                const uint32_t hi = *reinterpret_cast<const uint16_t *>(&table[o1]);
+                const uint32_t w2 = lo | (hi << 16);
+#pragma unroll
+                for (int m = 0; m < M; m++) acc[m][c & 1] = dot2(w2, X[m][wi][3 - c][i], acc[m][c & 1]);
+            };
+            static_for<4>([&](auto i_c) { static_for<4>([&](auto c_c) { gather_two(i_c, c_c); }); });
+        }
+    }
+}
+
+// Grid: ceil(N / R) workgroups of (64, S) threads; workgroup b owns rows
+// [b*R, b*R + R).  Host guarantees W % WPL == 0, S*64 <= THREADS,
+// R <= kGemvMaxRows, S*64*WPL >= W.  THREADS (256, 512 or 1024) only bounds the
+// workgroup size so that small workgroups may use more registers per lane
+// (M x WPL x 16 of them hold x).
+template <int BITS, int M, int WPL, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
+    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
+    const half_t *__restrict__ lut, half_t *__restrict__ out,
+    int N, int K, int R) {
+    constexpr int NC = 1 << BITS;
+    constexpr bool PAIR = GemvTable<BITS>::kPair;
+    constexpr int MAXS = THREADS / kWave;
+    typedef typename WordVec<WPL>::type wvec_t;
+    __shared__ __attribute__((aligned(16))) uint8_t tables[2][GemvTable<BITS>::kBytes];
+    __shared__ float partial[(MAXS > 1 ? MAXS : 1) * kGemvMaxRows * M];
+
+    const int lane = threadIdx.x;
+    const int s = __builtin_amdgcn_readfirstlane(threadIdx.y), S = blockDim.y;  // wave-uniform
+    const int W = K >> 5;
+    const size_t plane_stride = (size_t)N * W;
+
+    const int w0 = (s * kWave + lane) * WPL;
+    const bool valid = w0 < W;
+    const int wl = valid ? w0 : 0;  // lanes past the row end read word 0; their sums are dropped
+
+    uint32_t X[M][WPL][4][4];
+    load_activations<BITS, M, WPL>(x, K, wl, X);
+
+    const int row0 = blockIdx.x * R;
+    const int rows = min(R, N - row0);  // >= 1 by grid construction
 
     auto fetch_planes = [&](int row, wvec_t(&q)[BITS]) {
-        const uint32_t *p0 = qweight + (size_t)row * W + wl;
+        const uint32_t *p0 = qweight + (size_t)row * W;  // uniform: scalar base + lane offset
 #pragma unroll
-        for (int p = 0; p < BITS; p++) q[p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride);
+        for (int p = 0; p < BITS; p++) q[p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + (uint32_t)wl);
     };
 
     wvec_t qn[BITS];
-    LutRegs<BITS> ln;
-    if (row0 < N) {
-        fetch_planes(row0, qn);
-        ln = lut_fetch<BITS>(lut + (size_t)row0 * NC, lane);
-    }
+    TableRegs<BITS> tn;
+    fetch_planes(row0, qn);
+    if (s == 0) tn = table_fetch<BITS>(lut + (size_t)row0 * NC, lane);
 
-    for (int r = 0; r < R; r++) {
-        const int row = row0 + r * G;
-        if (row >= N) break;  // uniform per wave
+    auto do_row = [&](auto buf_c, int r) {
+        constexpr int BUF = decltype(buf_c)::value;
+        const int row = row0 + r;
         wvec_t q[BITS];
 #pragma unroll
         for (int p = 0; p < BITS; p++) q[p] = qn[p];
-        lut_stage<BITS>(ln, tab[r & 1], lane);
-        __builtin_amdgcn_wave_barrier();
-
-        const int next = row + G;
-        if (r + 1 < R && next < N) {
-            fetch_planes(next, qn);
-            ln = lut_fetch<BITS>(lut + (size_t)next * NC, lane);
+        if (s == 0) table_stage<BITS>(tn, tables[BUF], lane);
+        if (r + 1 < rows) {
+            fetch_planes(row + 1, qn);
+            if (s == 0) tn = table_fetch<BITS>(lut + (size_t)(row + 1) * NC, lane);
         }
+        // One barrier per row is enough: buffer BUF was last read two rows ago and
+        // every wave has passed the barrier of the row in between since.
+        if (S > 1) lds_barrier(); else __builtin_amdgcn_wave_barrier();
 
-        const half_t *t = tab[r & 1];
-        float acc[M];
+        float acc[M][2];
 #pragma unroll
-        for (int m = 0; m < M; m++) acc[m] = 0.f;
-#pragma unroll
-        for (int wi = 0; wi < WPL; wi++) {
-            uint32_t qq[BITS];
-#pragma unroll
-            for (int p = 0; p < BITS; p++) qq[p] = word_of<WPL>(q[p], wi);
-            uint32_t idx[8];
-            planes_to_indices<BITS>(qq, idx);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int sh = 8 * (3 - j);
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const uint16_t lo = __builtin_bit_cast(uint16_t, t[(idx[2 * i] >> sh) & 0xffu]);
-                    const uint16_t hi = __builtin_bit_cast(uint16_t, t[(idx[2 * i + 1] >> sh) & 0xffu]);
-                    const uint32_t wpair = (uint32_t)lo | ((uint32_t)hi << 16);
-#pragma unroll
-                    for (int m = 0; m < M; m++) acc[m] = dot2(wpair, X[m][wi][j][i], acc[m]);
-                }
-            }
-        }
+        for (int m = 0; m < M; m++) acc[m][0] = acc[m][1] = 0.f;
+        row_dot<BITS, M, WPL>(q, tables[BUF], X, acc);
 #pragma unroll
         for (int m = 0; m < M; m++) {
-            const float tot = wave_sum(valid ? acc[m] : 0.f);
+            const float tot = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
             if (lane == 0) {
                 if (S == 1) out[(size_t)m * N + row] = (half_t)tot;
-                else partial[((g * kGemvMaxRows + r) * S + s) * M + m] = tot;
+                else partial[(r * S + s) * M + m] = tot;
             }
         }
+    };
+
+    for (int r = 0; r < rows; r += 2) {
+        do_row(std::integral_constant<int, 0>{}, r);
+        if (r + 1 < rows) do_row(std::integral_constant<int, 1>{}, r + 1);
     }
 
     if (S > 1) {
         __syncthreads();
-        const int tid = (g * S + s) * kWave + lane;
-        const int nthreads = S * G * kWave;
-        for (int i = tid; i < G * R * M; i += nthreads) {
-            const int m = i % M, gr = i / M;
-            const int rr = gr % R, gg = gr / R;
-            const int row = blockIdx.x * (G * R) + rr * G + gg;
-            if (row < N) {
-                float tot = 0.f;
-                for (int ss = 0; ss < S; ss++) tot += partial[((gg * kGemvMaxRows + rr) * S + ss) * M + m];
-                out[(size_t)m * N + row] = (half_t)tot;
-            }
+        const int tid = s * kWave + lane;
+        for (int i = tid; i < rows * M; i += S * kWave) {
+            const int m = i % M, r = i / M;
+            float tot = 0.f;
+            for (int ss = 0; ss < S; ss++) tot += partial[(r * S + ss) * M + m];
+            out[(size_t)m * N + row0 + r] = (half_t)tot;
+        }
+    }
+}
+
+// "Flat" variant for M <= 2.  A workgroup is G independent row groups of S waves;
+// group g owns R consecutive rows (R = 1, 2 or 4, compile time) and issues every
+// global load it will ever need -- the planes of its R rows, their tables, the
+// activations -- before it computes anything, so the memory pipe is full from the
+// first cycle and there is no loop-carried prefetch.  Every table sits at a
+// compile-time LDS address: the code after the loads is instantiated once per
+// group index and selected by a uniform branch.  Several groups per workgroup
+// only serve to cut the number of workgroups the dispatcher has to launch.
+// Grid: ceil(N / (G*R)) workgroups of (64, S, G) threads; G*S*64 <= THREADS.
+template <int BITS, int M, int WPL, int R, int G, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
+    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
+    const half_t *__restrict__ lut, half_t *__restrict__ out, int N, int K) {
+    constexpr int NC = 1 << BITS;
+    constexpr int MAXS = THREADS / kWave / G;
+    typedef typename WordVec<WPL>::type wvec_t;
+    __shared__ __attribute__((aligned(16))) uint8_t tables[G][R][GemvTable<BITS>::kBytes];
+    __shared__ float partial[G][(MAXS > 1 ? MAXS : 1) * R * M];
+
+    // blockDim.x is the wave size, so threadIdx.y/z are wave-uniform: say so, to keep
+    // row addresses in scalar registers
+    const int lane = threadIdx.x;
+    const int s = __builtin_amdgcn_readfirstlane(threadIdx.y), S = blockDim.y;
+    const int g = __builtin_amdgcn_readfirstlane(threadIdx.z);
+    const int W = K >> 5;
+    const size_t plane_stride = (size_t)N * W;
+    const uint32_t w0 = (uint32_t)(s * kWave + lane) * WPL;
+    const bool valid = w0 < (uint32_t)W;
+    const uint32_t wl = valid ? w0 : 0u;  // lanes past the row end read word 0; their sums are dropped
+    const int row0 = (blockIdx.x * G + g) * R;
+
+    // rows past N (last workgroup only) re-read row N-1 and are not stored
+    wvec_t q[R][BITS];
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const uint32_t *p0 = qweight + (size_t)min(row0 + r, N - 1) * W;  // uniform per wave
+#pragma unroll
+        for (int p = 0; p < BITS; p++) q[r][p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + wl);
+    }
+    TableRegs<BITS> t[R];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        if (s == r % S) t[r] = table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane);
+
+    uint32_t X[M][WPL][4][4];
+    load_activations<BITS, M, WPL>(x, K, (int)wl, X);
+
+    float tot[R][M];
+    static_for<G>([&](auto g_c) {
+        constexpr int gi = decltype(g_c)::value;
+        if (g != gi) return;  // uniform per wave
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (s == r % S) table_stage<BITS>(t[r], tables[gi][r], lane);
+        if (S > 1) lds_barrier(); else __builtin_amdgcn_wave_barrier();
+        static_for<R>([&](auto r_c) {
+            constexpr int r = decltype(r_c)::value;
+            float acc[M][2];
+#pragma unroll
+            for (int m = 0; m < M; m++) acc[m][0] = acc[m][1] = 0.f;
+            row_dot<BITS, M, WPL>(q[r], tables[gi][r], X, acc);
+#pragma unroll
+            for (int m = 0; m < M; m++) tot[r][m] = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
+        });
+    });
+
+    if (S == 1) {
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int m = 0; m < M; m++)
+                    if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)tot[r][m];
+        }
+    } else {
+        // G == 1 whenever S > 1 (host), so the whole workgroup meets at these barriers
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int m = 0; m < M; m++) partial[g][(s * R + r) * M + m] = tot[r][m];
+        }
+        __syncthreads();
+        const int tid = s * kWave + lane;
+        if (tid < R * M) {
+            const int m = tid % M, r = tid / M;
+            float v = 0.f;
+            for (int ss = 0; ss < S; ss++) v += partial[g][(ss * R + r) * M + m];
+            if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)v;
         }
     }
 }

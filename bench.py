@@ -38,6 +38,12 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--table", default="", help="also write the per-layer table (markdown) to this file")
     ap.add_argument("--only-step", action="store_true", help="skip the per-kernel table (used under rocprofv3)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies, so a counter run has a kernel of known "
+                         "HBM traffic (read 256 MiB, write 256 MiB) to scale FETCH_SIZE / WRITE_SIZE with")
+    ap.add_argument("--eager", action="store_true",
+                    help="launch the timed steps one by one instead of replaying a HIP graph (rocprofv3 inflates "
+                         "the durations of graph-launched kernels, so profiles are taken in this mode)")
     return ap.parse_args()
 
 
@@ -90,23 +96,38 @@ def main():
 
     step_bytes = sum(synth.gemv_bytes(N, K, b, 1) for _, N, K in shapes for b in BITS)
 
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.int32, device="cuda")      # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)      # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- whole-step timing: the K steps are captured in one HIP graph so the host never starves the GPU
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         for i in range(args.warmup):
             step(i, side.cuda_stream)
         side.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            for i in range(args.steps):
-                step(args.warmup + i, torch.cuda.current_stream().cuda_stream)
-        graph.replay()                      # untimed: first replay pays graph upload
-        side.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record(side)
-        graph.replay()
-        e1.record(side)
+        if args.eager:
+            torch.cuda.synchronize()
+            e0.record(side)
+            for i in range(args.steps):
+                step(args.warmup + i, side.cuda_stream)
+            e1.record(side)
+        else:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(args.steps):
+                    step(args.warmup + i, torch.cuda.current_stream().cuda_stream)
+            graph.replay()                      # untimed: first replay pays graph upload
+            side.synchronize()
+            torch.cuda.synchronize()
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
         torch.cuda.synchronize()
         total_ms = e0.elapsed_time(e1)
     ms_per_step = total_ms / args.steps
@@ -143,8 +164,14 @@ def main():
     roofline = None
     if table:
         dom = max(table, key=lambda r: r["us"] * r["count_in_step"])
+        # HBM bytes per launch measured with rocprofv3 counters in separate runs (profiles/), if recorded
+        traffic = None
+        tfile = os.path.join(ROOT, "profiles", "gemv_kbit_hbm_traffic.json")
+        if os.path.exists(tfile):
+            with open(tfile) as f:
+                traffic = json.load(f)["bytes"].get(f"{dom['N']}x{dom['K']}:{dom['w_bits']}")
         roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": dom["frac"], "traffic": None,
+                    "frac": dom["frac"], "traffic": traffic,
                     "kernel": f"gemv_kbit_kernel<{dom['w_bits']},1,{dom['geometry']['wpl']},*> {dom['N']}x{dom['K']}",
                     "us_per_launch": dom["us"], "algorithmic_bytes_per_launch": dom["bytes"]}
 

@@ -60,10 +60,10 @@ const char *ap_strerror(int code);
 int ap_abi_version(void);
 
 /* Launch geometry the GEMV would use, for reports and tests: words per lane,
- * K-segments per workgroup, row groups per workgroup, rows per wave, grid size.
+ * K-segments (waves) per workgroup, rows per workgroup, grid size.
  * Returns AP_OK or the same argument errors as ap_matmul_kbit. */
 int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits,
-                            int *wpl, int *segments, int *groups, int *rows, int *grid);
+                            int *wpl, int *segments, int *rows, int *grid);
 
 #ifdef __cplusplus
 }

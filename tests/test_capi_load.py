@@ -69,7 +69,7 @@ def test_geometry_covers_rows_and_words():
             g = _capi.matmul_geometry(M, N, K, 4)
             W = K // 32
             assert g["segments"] * 64 * g["wpl"] >= W and W % g["wpl"] == 0
-            assert g["segments"] * g["groups"] <= 16 and 1 <= g["rows"] <= 8
-            assert g["grid"] * g["groups"] * g["rows"] >= N
+            assert g["segments"] <= 16 and 1 <= g["rows"] <= 16
+            assert g["grid"] * g["rows"] >= N and (g["grid"] - 1) * g["rows"] < N
     with pytest.raises(ValueError):
         _capi.matmul_geometry(1, 4, 32 * 64 * 2 * 17, 4)     # more K-segments than a workgroup holds
