@@ -63,7 +63,7 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     if (R < 1) R = 1;
     geo->flat = (M <= 2);
     if (geo->flat) {
-        R = R >= 4 ? 4 : (R >= 2 ? 2 : 1);
+        R = 1;  // one row per wave measured fastest (2 and 4 rows per wave lengthen the compute tail)
     } else if (R > kGemvMaxRows) {
         R = kGemvMaxRows;
     }
@@ -89,11 +89,7 @@ void launch_gemv_t(const GemvGeometry &geo, const uint16_t *x, const uint32_t *q
     const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
     half_t *oh = reinterpret_cast<half_t *>(out);
     if constexpr (M <= 2 && THREADS != 512) {
-        switch (geo.R) {
-            case 1: return launch_flat_g<BITS, M, WPL, 1, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
-            case 2: return launch_flat_g<BITS, M, WPL, 2, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
-            default: return launch_flat_g<BITS, M, WPL, 4, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
-        }
+        return launch_flat_g<BITS, M, WPL, 1, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
     } else if constexpr (M > 2) {
         const dim3 block(kWave, geo.S), grid(geo.grid);
         gemv_kbit_kernel<BITS, M, WPL, THREADS><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, N, K, geo.R);

@@ -62,19 +62,23 @@ __device__ __forceinline__ float dpp_add(float v) {
     return v + __builtin_bit_cast(float, moved);
 }
 
-// Sum over the 64 lanes of a wave; the total is returned in every lane.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add_rows(float v) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false);
+    return v + __builtin_bit_cast(float, moved);
+}
+
+// Sum over the 64 lanes of a wave in six DPP adds.  The total is valid in lanes
+// 48..63 only (kSumLane reads it); other lanes hold partial sums.
+constexpr int kSumLane = 63;
 __device__ __forceinline__ float wave_sum(float v) {
-    v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
-    v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
-    v = dpp_add<0x141>(v);  // row_half_mirror: lanes 0-3 <-> 7-4 within 8
-    v = dpp_add<0x140>(v);  // row_mirror: 0-7 <-> 15-8 within a row of 16
-    // every lane of a 16-lane row now holds its row's sum
-    const int vi = __builtin_bit_cast(int, v);
-    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 0));
-    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 16));
-    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 32));
-    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(vi, 48));
-    return (r0 + r1) + (r2 + r3);
+    v = dpp_add<0xB1>(v);            // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E>(v);            // quad_perm [2,3,0,1]
+    v = dpp_add<0x141>(v);           // row_half_mirror: lanes 0-3 <-> 7-4 within 8
+    v = dpp_add<0x140>(v);           // row_mirror: every lane of a 16-lane row holds the row sum
+    v = dpp_add_rows<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3
+    v = dpp_add_rows<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3: row 3 holds the total
+    return v;
 }
 
 // Copy one row's table of 2^BITS fp16 entries from global memory into this

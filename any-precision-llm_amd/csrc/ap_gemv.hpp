@@ -246,7 +246,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
 #pragma unroll
         for (int m = 0; m < M; m++) {
             const float tot = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
-            if (lane == 0) {
+            if (lane == kSumLane) {
                 if (S == 1) out[(size_t)m * N + row] = (half_t)tot;
                 else partial[(r * S + s) * M + m] = tot;
             }
@@ -301,7 +301,16 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
     const uint32_t wl = valid ? w0 : 0u;  // lanes past the row end read word 0; their sums are dropped
     const int row0 = (blockIdx.x * G + g) * R;
 
-    // rows past N (last workgroup only) re-read row N-1 and are not stored
+    // Issue order matters: the tables first (tiny; staging them to LDS then overlaps the
+    // plane loads -- issued last, the table was the last thing to arrive and cost 15-20 %),
+    // then the activations (L2 hits), then the planes (HBM).  Rows past N (last workgroup
+    // only) re-read row N-1 and are not stored.
+    TableRegs<BITS> t[R];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        if (s == r % S) t[r] = table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane);
+    uint32_t X[M][WPL][4][4];
+    load_activations<BITS, M, WPL>(x, K, (int)wl, X);
     wvec_t q[R][BITS];
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -309,13 +318,6 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
 #pragma unroll
         for (int p = 0; p < BITS; p++) q[r][p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + wl);
     }
-    TableRegs<BITS> t[R];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-        if (s == r % S) t[r] = table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane);
-
-    uint32_t X[M][WPL][4][4];
-    load_activations<BITS, M, WPL>(x, K, (int)wl, X);
 
     float tot[R][M];
     static_for<G>([&](auto g_c) {
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
     });
 
     if (S == 1) {
-        if (lane == 0) {
+        if (lane == kSumLane) {
 #pragma unroll
             for (int r = 0; r < R; r++)
 #pragma unroll
@@ -346,7 +348,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
         }
     } else {
         // G == 1 whenever S > 1 (host), so the whole workgroup meets at these barriers
-        if (lane == 0) {
+        if (lane == kSumLane) {
 #pragma unroll
             for (int r = 0; r < R; r++)
 #pragma unroll
