@@ -303,14 +303,13 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
 
     // Issue order matters: the tables first (tiny; staging them to LDS then overlaps the
     // plane loads -- issued last, the table was the last thing to arrive and cost 15-20 %),
-    // then the activations (L2 hits), then the planes (HBM).  Rows past N (last workgroup
-    // only) re-read row N-1 and are not stored.
+    // then the planes (HBM: the requests must go out at once), then the activations (L2
+    // hits; issued before the planes they cost up to 1 us at 3-5 bits).  Rows past N (last
+    // workgroup only) re-read row N-1 and are not stored.
     TableRegs<BITS> t[R];
 #pragma unroll
     for (int r = 0; r < R; r++)
         if (s == r % S) t[r] = table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane);
-    uint32_t X[M][WPL][4][4];
-    load_activations<BITS, M, WPL>(x, K, (int)wl, X);
     wvec_t q[R][BITS];
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -318,6 +317,8 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
 #pragma unroll
         for (int p = 0; p < BITS; p++) q[r][p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + wl);
     }
+    uint32_t X[M][WPL][4][4];
+    load_activations<BITS, M, WPL>(x, K, (int)wl, X);
 
     float tot[R][M];
     static_for<G>([&](auto g_c) {

@@ -5,7 +5,8 @@ Workload (the configuration the headline metric is quoted on): the seven linears
 Llama-2-7B decoder layer at batch 1 -- q,k,v,o 4096x4096, gate,up 11008x4096, down
 4096x11008 -- parent 8 bits, every w_bits in 3..8.  One "step" is one pass over those
 7 x 6 = 42 GEMVs.  Weights live in HBM before the timed region; consecutive steps walk a
-pool of distinct layers so that no launch finds its planes in the 256 MB last-level cache.
+pool of distinct weight sets (>= 1.5 GB of touched planes per shape) so that no launch finds
+its planes in the 256 MB last-level cache.
 
 Prints ONE JSON line: whole-step effective bandwidth (algorithmic bytes / time), the
 per-kernel roofline of the kernel that dominates the step, and the CPU baseline (the C
@@ -33,7 +34,9 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--pool", type=int, default=4, help="distinct decoder layers the steps rotate over")
+    ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
+    ap.add_argument("--pool-gb", type=float, default=1.5,
+                    help="per shape, GB of the three top planes over all weight sets of the pool")
     ap.add_argument("--kernel-reps", type=int, default=40, help="launches per (shape, w_bits) for the per-kernel table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--table", default="", help="also write the per-layer table (markdown) to this file")
@@ -47,19 +50,20 @@ def parse_args():
     return ap.parse_args()
 
 
-class Layer:
-    """Device-resident synthetic linear: uniform parent codes are uniform plane bits, so the
-    planes are drawn directly as random words; tables are ascending N(0, 0.02) draws."""
+class WeightPool:
+    """`sets` device-resident synthetic linears of one shape.  Uniform parent codes are
+    uniform plane bits, so planes are drawn directly as random words; tables are ascending
+    N(0, 0.02) draws (std 0.02), one per set and precision."""
 
-    def __init__(self, torch, N, K, gen):
-        self.N, self.K = N, K
-        self.qweight = torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda",
+    def __init__(self, torch, N, K, sets, gen):
+        self.N, self.K, self.sets = N, K, sets
+        self.qweight = torch.randint(-2**31, 2**31 - 1, (sets, 8, N, K // 32), dtype=torch.int32, device="cuda",
                                      generator=gen)
         self.luts = {}
         for b in BITS:
-            t = torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02
-            self.luts[b] = torch.sort(t, dim=1).values.to(torch.float16).contiguous()
-        self.out = torch.empty((1, N), dtype=torch.float16, device="cuda")
+            t = torch.randn((sets, N, 1 << b), device="cuda", generator=gen) * 0.02
+            self.luts[b] = torch.sort(t, dim=2).values.to(torch.float16).contiguous()
+        self.out = torch.empty((8, N), dtype=torch.float16, device="cuda")
 
 
 def main():
@@ -78,21 +82,35 @@ def main():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
     shapes = [(n, N, K) for n, N, K in synth.LLAMA2_7B_LAYER]
+    uniq = {}
+    for idx, (name, N, K) in enumerate(shapes):
+        uniq.setdefault((N, K), []).append(idx)
 
-    pool = [[Layer(torch, N, K, gen) for _, N, K in shapes] for _ in range(args.pool)]
+    # Cold-cache discipline: every launch reads a weight set that no recent launch touched.  Per
+    # shape the pool holds enough sets that even the 3 top planes of all sets exceed
+    # `--pool-gb` (default 1.5 GB, six times the 256 MB last-level cache).
+    pools = {}
+    for (N, K), idxs in uniq.items():
+        need = int(args.pool_gb * 1e9 / (3 * N * K / 8)) + 1
+        sets = max(need, len(idxs) * args.pool)
+        pools[(N, K)] = WeightPool(torch, N, K, sets, gen)
     xs = {K: torch.randn((1, K), device="cuda", generator=gen).to(torch.float16) for K in {K for _, _, K in shapes}}
     torch.cuda.synchronize()
+    cursor = {k: 0 for k in pools}
 
-    def launch(layer: Layer, b: int, stream: int):
-        rc = lib.ap_matmul_kbit(xs[layer.K].data_ptr(), layer.qweight.data_ptr(), layer.luts[b].data_ptr(),
-                                layer.out.data_ptr(), 1, layer.N, layer.K, b, stream)
+    def launch(N: int, K: int, b: int, stream: int):
+        """One GEMV on the next weight set of its shape."""
+        P = pools[(N, K)]
+        j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
+        rc = lib.ap_matmul_kbit(xs[K].data_ptr(), P.qweight[j].data_ptr(), P.luts[b][j].data_ptr(),
+                                P.out.data_ptr(), 1, N, K, b, stream)
         if rc != 0:
             raise RuntimeError(_capi.strerror(rc))
 
     def step(i: int, stream: int):
         for b in BITS:
-            for layer in pool[i % args.pool]:
-                launch(layer, b, stream)
+            for _, N, K in shapes:
+                launch(N, K, b, stream)
 
     step_bytes = sum(synth.gemv_bytes(N, K, b, 1) for _, N, K in shapes for b in BITS)
 
@@ -136,17 +154,13 @@ def main():
     # ---- per-kernel table: each (shape, w_bits) alone, rotating over the pool (cold planes)
     table = []
     if not args.only_step:
-        uniq = {}
-        for idx, (name, N, K) in enumerate(shapes):
-            uniq.setdefault((N, K), []).append(idx)
         with torch.cuda.stream(side):
             for (N, K), idxs in uniq.items():
-                layers = [pool[p][i] for p in range(args.pool) for i in idxs]
                 for b in BITS:
                     g = torch.cuda.CUDAGraph()
                     with torch.cuda.graph(g, stream=side):
                         for r in range(args.kernel_reps):
-                            launch(layers[r % len(layers)], b, torch.cuda.current_stream().cuda_stream)
+                            launch(N, K, b, torch.cuda.current_stream().cuda_stream)
                     g.replay()
                     side.synchronize()
                     a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -207,7 +221,8 @@ def main():
         "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate", "data": "synthetic",
         "config": {"workload": "Llama-2-7B decoder-layer linear set (q,k,v,o 4096x4096; gate,up 11008x4096; "
                                "down 4096x11008), batch 1, parent 8 bits, w_bits 3..8 = 42 GEMVs per step",
-                   "pool_layers": args.pool, "bytes_per_step": step_bytes,
+                   "weight_sets_per_shape": {f"{N}x{K}": P.sets for (N, K), P in pools.items()},
+                   "bytes_per_step": step_bytes,
                    "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline, "cpu_baseline": cpu, "layers": table,
     }
