@@ -67,7 +67,9 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     if (R < 1) R = 1;
     geo->flat = (M <= 2);
     if (geo->flat) {
-        R = 1;  // one row per wave measured fastest (2 and 4 rows per wave lengthen the compute tail)
+        // one row per wave until that would launch more than target_waves waves, then two (the
+        // second row reuses the activation registers); four lengthen the compute tail
+        R = R >= 2 ? 2 : 1;
     } else if (R > kGemvMaxRows) {
         R = kGemvMaxRows;
     }
@@ -93,6 +95,7 @@ void launch_gemv_t(const GemvGeometry &geo, const uint16_t *x, const uint32_t *q
     const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
     half_t *oh = reinterpret_cast<half_t *>(out);
     if constexpr (M <= 2 && THREADS != 512) {
+        if (geo.R == 2) return launch_flat_g<BITS, M, WPL, 2, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
         return launch_flat_g<BITS, M, WPL, 1, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
     } else if constexpr (M > 2) {
         const dim3 block(kWave, geo.S), grid(geo.grid);
