@@ -43,7 +43,7 @@ __global__ __launch_bounds__(kDequantWaves * kWave) void dequant_kbit_kernel(
         for (int w = lane; w < W; w += kWave) {
             uint32_t q[BITS];
 #pragma unroll
-            for (int p = 0; p < BITS; p++) q[p] = wrow[p * plane_stride + w];
+            for (int p = 0; p < BITS; p++) q[p] = __builtin_nontemporal_load(wrow + p * plane_stride + w);
             uint32_t idx[8];
             planes_to_indices<BITS>(q, idx);
 #pragma unroll

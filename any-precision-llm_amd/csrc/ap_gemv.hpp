@@ -192,7 +192,6 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
     const half_t *__restrict__ lut, half_t *__restrict__ out,
     int N, int K, int R) {
     constexpr int NC = 1 << BITS;
-    constexpr bool PAIR = GemvTable<BITS>::kPair;
     constexpr int MAXS = THREADS / kWave;
     typedef typename WordVec<WPL>::type wvec_t;
     __shared__ __attribute__((aligned(16))) uint8_t tables[2][GemvTable<BITS>::kBytes];
@@ -216,7 +215,8 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
     auto fetch_planes = [&](int row, wvec_t(&q)[BITS]) {
         const uint32_t *p0 = qweight + (size_t)row * W;  // uniform: scalar base + lane offset
 #pragma unroll
-        for (int p = 0; p < BITS; p++) q[p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + (uint32_t)wl);
+        for (int p = 0; p < BITS; p++)
+            q[p] = __builtin_nontemporal_load(reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + (uint32_t)wl));
     };
 
     wvec_t qn[BITS];
@@ -315,7 +315,8 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
     for (int r = 0; r < R; r++) {
         const uint32_t *p0 = qweight + (size_t)min(row0 + r, N - 1) * W;  // uniform per wave
 #pragma unroll
-        for (int p = 0; p < BITS; p++) q[r][p] = *reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + wl);
+        for (int p = 0; p < BITS; p++)  // streamed once: non-temporal, so x and the tables keep their cache lines
+            q[r][p] = __builtin_nontemporal_load(reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + wl));
     }
     uint32_t X[M][WPL][4][4];
     load_activations<BITS, M, WPL>(x, K, (int)wl, X);
