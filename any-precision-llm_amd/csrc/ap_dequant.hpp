@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kDequantWaves * kWave) void dequant_kbit_kernel(
                     const uint16_t hi = __builtin_bit_cast(uint16_t, tab[(idx[2 * i + 1] >> sh) & 0xffu]);
                     v[i] = (uint32_t)lo | ((uint32_t)hi << 16);
                 }
-                *reinterpret_cast<u32x4 *>(orow + group_base(w, j, K)) = v;
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(orow + group_base(w, j, K)));
             }
         }
     }
