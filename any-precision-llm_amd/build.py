@@ -14,6 +14,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
+OBJDIR = os.path.join(HERE, "build")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 
 HIP_LIB = os.path.join(LIBDIR, "libanyprec_hip.so")
@@ -34,19 +35,33 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def build_hip(verbose: bool = False, extra_flags=()) -> str:
-    os.makedirs(LIBDIR, exist_ok=True)
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, "-I", CSRC,
-           os.path.join(CSRC, "ap_capi.hip"), "-o", HIP_LIB]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     # the host pass does not know the packed-fp32 feature and says so; drop that line
     out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 7) -> str:
+    """One object per GEMV bit-width (compiled in parallel) + the C ABI, linked into the .so."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    os.makedirs(OBJDIR, exist_ok=True)
+    os.makedirs(LIBDIR, exist_ok=True)
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"] + list(extra_flags) + ["-I", INCLUDE, "-I", CSRC, "-c"]
+    units = [(os.path.join(CSRC, "ap_capi.hip"), os.path.join(OBJDIR, "ap_capi.o"), [])]
+    for b in range(3, 9):
+        units.append((os.path.join(CSRC, "ap_gemv_inst.hip"), os.path.join(OBJDIR, f"ap_gemv_b{b}.o"), [f"-DAP_BITS={b}"]))
+    hipcc = _hipcc()
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(lambda u: _run([hipcc, *compile_flags, *u[2], u[0], "-o", u[1]], verbose), units))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *[u[1] for u in units], "-o", HIP_LIB],
+         verbose)
     return HIP_LIB
 
 

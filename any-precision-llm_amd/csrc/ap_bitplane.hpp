@@ -14,6 +14,7 @@
 #include <stdint.h>
 
 #if defined(__HIPCC__)
+#include <hip/hip_runtime.h>
 #define AP_HD __host__ __device__ __forceinline__
 #else
 #define AP_HD inline

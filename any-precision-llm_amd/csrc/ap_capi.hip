@@ -5,7 +5,7 @@
 
 #include "anyprec_hip.h"
 #include "ap_dequant.hpp"
-#include "ap_gemv.hpp"
+#include "ap_gemv_launch.hpp"
 
 namespace {
 
@@ -43,11 +43,6 @@ int check_common(int N, int K, int w_bits) {
     return AP_OK;
 }
 
-struct GemvGeometry {
-    int wpl, S, R, G, grid;
-    bool flat;  // everything-prefetched kernel (M <= 2), R in {1, 2, 4}
-};
-
 int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     const int rc = check_common(N, K, w_bits);
     if (rc != AP_OK) return rc;
@@ -63,79 +58,16 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     const int seg = kWave * wpl;
     const int S = (W + seg - 1) / seg;
     if (S > kGemvMaxSeg) return AP_ELIMIT;
+    // One row per workgroup until that would launch more than target_waves waves, then two
+    // (the second row reuses the activation registers; more rows lengthen the compute
+    // tail).  From M = 3 on the activations are the larger load: always two rows.
     int R = t.force_rows > 0 ? t.force_rows : (int)(((long long)N * S + t.target_waves - 1) / t.target_waves);
-    if (R < 1) R = 1;
-    geo->flat = (M <= 2);
-    if (geo->flat) {
-        // one row per wave until that would launch more than target_waves waves, then two (the
-        // second row reuses the activation registers); four lengthen the compute tail
-        R = R >= 2 ? 2 : 1;
-    } else if (R > kGemvMaxRows) {
-        R = kGemvMaxRows;
-    }
-    // row groups per workgroup (packing several measured no faster than one)
-    geo->G = 1;
+    R = (R >= 2 || M > 2) ? 2 : 1;
     geo->wpl = wpl;
     geo->S = S;
     geo->R = R;
-    geo->grid = (N + R * geo->G - 1) / (R * geo->G);
+    geo->grid = (N + R - 1) / R;
     return AP_OK;
-}
-
-template <int BITS, int M, int WPL, int R, int THREADS>
-void launch_flat_g(const GemvGeometry &geo, const half_t *x, const uint32_t *qweight, const half_t *lut,
-                   half_t *out, int N, int K, hipStream_t stream) {
-    const dim3 block(kWave, geo.S, geo.G), grid(geo.grid);
-    gemv_kbit_flat_kernel<BITS, M, WPL, R, 1, THREADS><<<grid, block, 0, stream>>>(x, qweight, lut, out, N, K);
-}
-
-template <int BITS, int M, int WPL, int THREADS>
-void launch_gemv_t(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
-                   uint16_t *out, int N, int K, hipStream_t stream) {
-    const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
-    half_t *oh = reinterpret_cast<half_t *>(out);
-    if constexpr (M <= 2 && THREADS != 512) {
-        if (geo.R == 2) return launch_flat_g<BITS, M, WPL, 2, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
-        return launch_flat_g<BITS, M, WPL, 1, THREADS>(geo, xh, qweight, lh, oh, N, K, stream);
-    } else if constexpr (M > 2) {
-        const dim3 block(kWave, geo.S), grid(geo.grid);
-        gemv_kbit_kernel<BITS, M, WPL, THREADS><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, N, K, geo.R);
-    }
-}
-
-// Smallest workgroup bound that holds S waves: leaves the most registers per lane.
-template <int BITS, int M, int WPL>
-void launch_gemv(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
-                 uint16_t *out, int N, int K, hipStream_t stream) {
-    if (geo.S <= 4) return launch_gemv_t<BITS, M, WPL, 256>(geo, x, qweight, lut, out, N, K, stream);
-    if constexpr (M > 2) {
-        if (geo.S <= 8) return launch_gemv_t<BITS, M, WPL, 512>(geo, x, qweight, lut, out, N, K, stream);
-    }
-    launch_gemv_t<BITS, M, WPL, 1024>(geo, x, qweight, lut, out, N, K, stream);
-}
-
-template <int BITS, int M>
-void launch_gemv_wpl(const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
-                     uint16_t *out, int N, int K, hipStream_t stream) {
-    if constexpr (M <= 2) {
-        if (geo.wpl == 2) return launch_gemv<BITS, M, 2>(geo, x, qweight, lut, out, N, K, stream);
-    }
-    launch_gemv<BITS, M, 1>(geo, x, qweight, lut, out, N, K, stream);
-}
-
-template <int BITS>
-void launch_gemv_m(int M, const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight,
-                   const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream) {
-    switch (M) {
-        case 1: return launch_gemv_wpl<BITS, 1>(geo, x, qweight, lut, out, N, K, stream);
-        case 2: return launch_gemv_wpl<BITS, 2>(geo, x, qweight, lut, out, N, K, stream);
-        case 3: return launch_gemv_wpl<BITS, 3>(geo, x, qweight, lut, out, N, K, stream);
-        case 4: return launch_gemv_wpl<BITS, 4>(geo, x, qweight, lut, out, N, K, stream);
-        case 5: return launch_gemv_wpl<BITS, 5>(geo, x, qweight, lut, out, N, K, stream);
-        case 6: return launch_gemv_wpl<BITS, 6>(geo, x, qweight, lut, out, N, K, stream);
-        case 7: return launch_gemv_wpl<BITS, 7>(geo, x, qweight, lut, out, N, K, stream);
-        default: return launch_gemv_wpl<BITS, 8>(geo, x, qweight, lut, out, N, K, stream);
-    }
 }
 
 template <int BITS>
@@ -211,12 +143,12 @@ int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *l
     if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
     switch (w_bits) {
-        case 3: launch_gemv_m<3>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 4: launch_gemv_m<4>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 5: launch_gemv_m<5>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 6: launch_gemv_m<6>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 7: launch_gemv_m<7>(M, geo, x, qweight, lut, out, N, K, st); break;
-        default: launch_gemv_m<8>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 3: launch_gemv<3>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 4: launch_gemv<4>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 5: launch_gemv<5>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 6: launch_gemv<6>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 7: launch_gemv<7>(M, geo, x, qweight, lut, out, N, K, st); break;
+        default: launch_gemv<8>(M, geo, x, qweight, lut, out, N, K, st); break;
     }
     return launch_status();
 }

@@ -5,38 +5,31 @@
 // (any_precision/modules/kernels/matmul.cuh:16-167); the reference sums in
 // fp16, this kernel in fp32.
 //
-// The kernel is bound by VALU and LDS-gather issue rather than by HBM at low
-// bit-widths (a table lookup per weight), so the design minimises instructions
-// per weight:
-//   * A workgroup is S waves that walk the same R consecutive rows together;
-//     wave s owns K-segment s (64*WPL consecutive words = 2048*WPL elements).
-//     One row is in flight per workgroup, so the row's table sits at a
-//     compile-time LDS address and a gather address is a single SDWA
-//     byte-extract-and-shift.
-//   * The activations a lane needs are the same for every row: they are loaded
-//     once into registers, already permuted into the order the packed layout
-//     scatters elements.
-//   * Per row a lane streams WPL words per plane (one load per plane, a wave
-//     covers 256*WPL contiguous bytes), rebuilds its indices with a butterfly
-//     transpose in registers, gathers from LDS and feeds v_dot2c_f32_f16.
+// Per weight the path costs a table lookup, so besides HBM it loads the VALU and the LDS
+// gather pipe; the design minimises instructions per weight and keeps every wave short:
+//   * A workgroup is the S waves of R consecutive rows; wave s owns K-segment s (64*WPL
+//     consecutive words = 2048*WPL elements).  The row's table sits at a compile-time LDS
+//     address and a gather address is a single SDWA byte-extract-and-shift.
+//   * The activations a lane needs are the same for every row: they are loaded into
+//     registers, already permuted into the order the packed layout scatters elements.
+//   * Per row a lane streams WPL words per plane (one load per plane, a wave covers
+//     256*WPL contiguous bytes), rebuilds its indices with a butterfly transpose in
+//     registers, gathers from LDS and feeds v_dot2c_f32_f16.
 //   * 3 and 4 bits use a pair table (reference idea: matmul.cuh:24,41-49,
-//     dequant.cuh:13-30,56-67): 4^b entries of two fp16 (w[e], w[e+4]), one
-//     32-bit gather per two weights and no packing.  5..8 bits gather single
-//     fp16 entries and pack two of them per dot2.
-//   * Next row's planes and table are prefetched while the current row is
-//     computed; tables are double-buffered so one barrier per row suffices.
-//   * Lane partials are summed with DPP; when S > 1 the segment partials of a
-//     row meet in LDS and are added in a fixed order: results are deterministic.
+//     dequant.cuh:13-30,56-67): 4^b entries of two fp16 (w[e], w[e+4]), one 32-bit gather
+//     per two weights and no packing.  5..8 bits gather single fp16 entries and pack two of
+//     them per dot2.
+//   * Lane partials are summed with DPP; when S > 1 the segment partials of a row meet in
+//     LDS and are added in a fixed order: results are deterministic.
 #pragma once
 #include <type_traits>
 
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
+#include "ap_gemv_launch.hpp"
 
 namespace ap {
 
-constexpr int kGemvMaxSeg = 16;   // K-segments (waves) per workgroup
-constexpr int kGemvMaxRows = 16;  // rows per workgroup upper bound (R)
 
 template <int BITS>
 struct GemvTable {
@@ -181,125 +174,34 @@ __device__ __forceinline__ void row_dot(const typename WordVec<WPL>::type (&q)[B
     }
 }
 
-// Grid: ceil(N / R) workgroups of (64, S) threads; workgroup b owns rows
-// [b*R, b*R + R).  Host guarantees W % WPL == 0, S*64 <= THREADS,
-// R <= kGemvMaxRows, S*64*WPL >= W.  THREADS (256, 512 or 1024) only bounds the
-// workgroup size so that small workgroups may use more registers per lane
-// (M x WPL x 16 of them hold x).
-template <int BITS, int M, int WPL, int THREADS>
+// The GEMV kernel.  A workgroup is the S waves of R consecutive rows (R = 1 or 2,
+// compile time).  Every wave issues all the global loads it will ever need -- the tables,
+// the planes of its R rows, its activations -- before it computes anything, so the
+// memory pipe is full from the first cycle and there is no loop-carried prefetch.  Every
+// table sits at a compile-time LDS address.
+// Grid: ceil(N / R) workgroups of (64, S) threads; S*64 <= THREADS.  THREADS (256, 512 or
+// 1024) only bounds the workgroup size, so that small workgroups may use more registers
+// per lane (M x WPL x 16 of them hold the activations).
+template <int BITS, int M, int WPL, int R, int THREADS>
 __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
-    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
-    const half_t *__restrict__ lut, half_t *__restrict__ out,
-    int N, int K, int R) {
-    constexpr int NC = 1 << BITS;
-    constexpr int MAXS = THREADS / kWave;
-    typedef typename WordVec<WPL>::type wvec_t;
-    __shared__ __attribute__((aligned(16))) uint8_t tables[2][GemvTable<BITS>::kBytes];
-    __shared__ float partial[(MAXS > 1 ? MAXS : 1) * kGemvMaxRows * M];
-
-    const int lane = threadIdx.x;
-    const int s = __builtin_amdgcn_readfirstlane(threadIdx.y), S = blockDim.y;  // wave-uniform
-    const int W = K >> 5;
-    const size_t plane_stride = (size_t)N * W;
-
-    const int w0 = (s * kWave + lane) * WPL;
-    const bool valid = w0 < W;
-    const int wl = valid ? w0 : 0;  // lanes past the row end read word 0; their sums are dropped
-
-    uint32_t X[M][WPL][4][4];
-    load_activations<BITS, M, WPL>(x, K, wl, X);
-
-    const int row0 = blockIdx.x * R;
-    const int rows = min(R, N - row0);  // >= 1 by grid construction
-
-    auto fetch_planes = [&](int row, wvec_t(&q)[BITS]) {
-        const uint32_t *p0 = qweight + (size_t)row * W;  // uniform: scalar base + lane offset
-#pragma unroll
-        for (int p = 0; p < BITS; p++)
-            q[p] = __builtin_nontemporal_load(reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + (uint32_t)wl));
-    };
-
-    wvec_t qn[BITS];
-    TableRegs<BITS> tn;
-    fetch_planes(row0, qn);
-    if (s == 0) tn = table_fetch<BITS>(lut + (size_t)row0 * NC, lane);
-
-    auto do_row = [&](auto buf_c, int r) {
-        constexpr int BUF = decltype(buf_c)::value;
-        const int row = row0 + r;
-        wvec_t q[BITS];
-#pragma unroll
-        for (int p = 0; p < BITS; p++) q[p] = qn[p];
-        if (s == 0) table_stage<BITS>(tn, tables[BUF], lane);
-        if (r + 1 < rows) {
-            fetch_planes(row + 1, qn);
-            if (s == 0) tn = table_fetch<BITS>(lut + (size_t)(row + 1) * NC, lane);
-        }
-        // One barrier per row is enough: buffer BUF was last read two rows ago and
-        // every wave has passed the barrier of the row in between since.
-        if (S > 1) lds_barrier(); else __builtin_amdgcn_wave_barrier();
-
-        float acc[M][2];
-#pragma unroll
-        for (int m = 0; m < M; m++) acc[m][0] = acc[m][1] = 0.f;
-        row_dot<BITS, M, WPL>(q, tables[BUF], X, acc);
-#pragma unroll
-        for (int m = 0; m < M; m++) {
-            const float tot = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
-            if (lane == kSumLane) {
-                if (S == 1) out[(size_t)m * N + row] = (half_t)tot;
-                else partial[(r * S + s) * M + m] = tot;
-            }
-        }
-    };
-
-    for (int r = 0; r < rows; r += 2) {
-        do_row(std::integral_constant<int, 0>{}, r);
-        if (r + 1 < rows) do_row(std::integral_constant<int, 1>{}, r + 1);
-    }
-
-    if (S > 1) {
-        __syncthreads();
-        const int tid = s * kWave + lane;
-        for (int i = tid; i < rows * M; i += S * kWave) {
-            const int m = i % M, r = i / M;
-            float tot = 0.f;
-            for (int ss = 0; ss < S; ss++) tot += partial[(r * S + ss) * M + m];
-            out[(size_t)m * N + row0 + r] = (half_t)tot;
-        }
-    }
-}
-
-// "Flat" variant for M <= 2.  A workgroup is G independent row groups of S waves;
-// group g owns R consecutive rows (R = 1, 2 or 4, compile time) and issues every
-// global load it will ever need -- the planes of its R rows, their tables, the
-// activations -- before it computes anything, so the memory pipe is full from the
-// first cycle and there is no loop-carried prefetch.  Every table sits at a
-// compile-time LDS address: the code after the loads is instantiated once per
-// group index and selected by a uniform branch.  Several groups per workgroup
-// only serve to cut the number of workgroups the dispatcher has to launch.
-// Grid: ceil(N / (G*R)) workgroups of (64, S, G) threads; G*S*64 <= THREADS.
-template <int BITS, int M, int WPL, int R, int G, int THREADS>
-__global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
     const half_t *__restrict__ lut, half_t *__restrict__ out, int N, int K) {
     constexpr int NC = 1 << BITS;
-    constexpr int MAXS = THREADS / kWave / G;
+    constexpr int MAXS = THREADS / kWave;
     typedef typename WordVec<WPL>::type wvec_t;
-    __shared__ __attribute__((aligned(16))) uint8_t tables[G][R][GemvTable<BITS>::kBytes];
-    __shared__ float partial[G][(MAXS > 1 ? MAXS : 1) * R * M];
+    __shared__ __attribute__((aligned(16))) uint8_t tables[R][GemvTable<BITS>::kBytes];
+    __shared__ float partial[MAXS * R * M];
 
-    // blockDim.x is the wave size, so threadIdx.y/z are wave-uniform: say so, to keep
-    // row addresses in scalar registers
+    // blockDim.x is the wave size, so threadIdx.y is wave-uniform: say so, to keep row
+    // addresses in scalar registers
     const int lane = threadIdx.x;
     const int s = __builtin_amdgcn_readfirstlane(threadIdx.y), S = blockDim.y;
-    const int g = __builtin_amdgcn_readfirstlane(threadIdx.z);
     const int W = K >> 5;
     const size_t plane_stride = (size_t)N * W;
     const uint32_t w0 = (uint32_t)(s * kWave + lane) * WPL;
     const bool valid = w0 < (uint32_t)W;
     const uint32_t wl = valid ? w0 : 0u;  // lanes past the row end read word 0; their sums are dropped
-    const int row0 = (blockIdx.x * G + g) * R;
+    const int row0 = blockIdx.x * R;
 
     // Issue order matters: the tables first (tiny; staging them to LDS then overlaps the
     // plane loads -- issued last, the table was the last thing to arrive and cost 15-20 %),
@@ -321,23 +223,20 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
     uint32_t X[M][WPL][4][4];
     load_activations<BITS, M, WPL>(x, K, (int)wl, X);
 
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        if (s == r % S) table_stage<BITS>(t[r], tables[r], lane);
+    if (S > 1) lds_barrier(); else __builtin_amdgcn_wave_barrier();
+
     float tot[R][M];
-    static_for<G>([&](auto g_c) {
-        constexpr int gi = decltype(g_c)::value;
-        if (g != gi) return;  // uniform per wave
+    static_for<R>([&](auto r_c) {
+        constexpr int r = decltype(r_c)::value;
+        float acc[M][2];
 #pragma unroll
-        for (int r = 0; r < R; r++)
-            if (s == r % S) table_stage<BITS>(t[r], tables[gi][r], lane);
-        if (S > 1) lds_barrier(); else __builtin_amdgcn_wave_barrier();
-        static_for<R>([&](auto r_c) {
-            constexpr int r = decltype(r_c)::value;
-            float acc[M][2];
+        for (int m = 0; m < M; m++) acc[m][0] = acc[m][1] = 0.f;
+        row_dot<BITS, M, WPL>(q[r], tables[r], X, acc);
 #pragma unroll
-            for (int m = 0; m < M; m++) acc[m][0] = acc[m][1] = 0.f;
-            row_dot<BITS, M, WPL>(q[r], tables[gi][r], X, acc);
-#pragma unroll
-            for (int m = 0; m < M; m++) tot[r][m] = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
-        });
+        for (int m = 0; m < M; m++) tot[r][m] = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
     });
 
     if (S == 1) {
@@ -349,19 +248,18 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_flat_kernel(
                     if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)tot[r][m];
         }
     } else {
-        // G == 1 whenever S > 1 (host), so the whole workgroup meets at these barriers
         if (lane == kSumLane) {
 #pragma unroll
             for (int r = 0; r < R; r++)
 #pragma unroll
-                for (int m = 0; m < M; m++) partial[g][(s * R + r) * M + m] = tot[r][m];
+                for (int m = 0; m < M; m++) partial[(s * R + r) * M + m] = tot[r][m];
         }
         __syncthreads();
         const int tid = s * kWave + lane;
-        if (tid < R * M) {
+        if (tid < R * M) {  // S >= 2 waves hold at least 128 threads >= R * M
             const int m = tid % M, r = tid / M;
             float v = 0.f;
-            for (int ss = 0; ss < S; ss++) v += partial[g][(ss * R + r) * M + m];
+            for (int ss = 0; ss < S; ss++) v += partial[(ss * R + r) * M + m];
             if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)v;
         }
     }

@@ -1,0 +1,31 @@
+// Host-side launch interface of the GEMV kernels.  The kernels of one bit-width are
+// compiled in their own translation unit (ap_gemv_inst.hip with -DAP_BITS=b) so that the
+// six bit-widths build in parallel; ap_capi.hip only sees these declarations.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ap {
+
+constexpr int kGemvMaxSeg = 16;  // K-segments (waves) per workgroup
+
+struct GemvGeometry {
+    int wpl;   // words per lane per plane (1 or 2)
+    int S;     // K-segments = waves per workgroup
+    int R;     // rows per workgroup (1 or 2)
+    int grid;  // workgroups
+};
+
+// Launches gemv_kbit_kernel<BITS, M, geo.wpl, geo.R, *> on `stream`.  1 <= M <= 8.
+template <int BITS>
+void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight,
+                 const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream);
+
+extern template void launch_gemv<3>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+extern template void launch_gemv<4>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+extern template void launch_gemv<5>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+extern template void launch_gemv<6>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+extern template void launch_gemv<7>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+extern template void launch_gemv<8>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+
+}  // namespace ap
