@@ -31,6 +31,8 @@ lib.ap_dequant_kbit.argtypes = [_vp, _vp, _vp, _ci, _ci, _ci, _vp]
 lib.ap_dequant_kbit.restype = _ci
 lib.ap_matmul_kbit.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 lib.ap_matmul_kbit.restype = _ci
+lib.ap_gemm_kbit.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
+lib.ap_gemm_kbit.restype = _ci
 _pi = ctypes.POINTER(ctypes.c_int)
 lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi]
 lib.ap_matmul_kbit_geometry.restype = _ci
@@ -40,7 +42,9 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
         f"{LIB_PATH} has ABI version {lib.ap_abi_version()}, this binding needs {AP_ABI_VERSION}: rebuild it"
     )
 
-EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_geometry")
+EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_gemm_kbit",
+           "ap_matmul_kbit_geometry")
+GEMM_MAX_M = 128
 
 
 def strerror(code: int) -> str:

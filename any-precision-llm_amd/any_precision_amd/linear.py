@@ -4,8 +4,9 @@
 Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]``,
 ``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
 ``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
-Batch dispatch follows the reference (:60-64): more than 8 activation rows ->
-``dequant_kbit`` + ``torch.matmul``, otherwise ``matmul_kbit``.
+Batch dispatch: up to 8 activation rows -> ``matmul_kbit`` as in the reference (:60-64);
+9 .. ``GEMM_MAX_M`` rows -> the fused ``gemm_kbit``; beyond -> ``dequant_kbit`` +
+``torch.matmul`` as in the reference.
 """
 from __future__ import annotations
 
@@ -13,9 +14,9 @@ import torch
 import torch.nn as nn
 
 try:
-    from any_precision_ext import matmul_kbit, dequant_kbit
+    from any_precision_ext import matmul_kbit, dequant_kbit, gemm_kbit, GEMM_MAX_M
 except ModuleNotFoundError:
-    matmul_kbit, dequant_kbit = None, None
+    matmul_kbit, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, 0
 
 
 class AnyPrecisionLinear(nn.Module):
@@ -59,11 +60,14 @@ class AnyPrecisionLinear(nn.Module):
     def forward(self, x, **kwargs):
         w_bits = kwargs["precision"] if "precision" in kwargs else self.precision
         lut = self._buffers[f"lut{w_bits}"]
-        if x.numel() // x.shape[-1] > 8:
+        rows = x.numel() // x.shape[-1]
+        if rows <= 8:
+            x = matmul_kbit(x, self.qweight, lut, w_bits)
+        elif rows <= GEMM_MAX_M and x.is_contiguous():
+            x = gemm_kbit(x, self.qweight, lut, w_bits)      # fused dequant -> MFMA, weight never materialised
+        else:
             weight = dequant_kbit(self.qweight, lut, w_bits)
             x = torch.matmul(x, weight.T)
-        else:
-            x = matmul_kbit(x, self.qweight, lut, w_bits)
         if self.bias is not None:
             x += self.bias
         return x

@@ -5,6 +5,10 @@ signatures, same result shapes and dtypes.
     matmul_kbit(in, qweight, lut, w_bits) -> Tensor   main.cu:93-143
     dequant_kbit(qweight, lut, w_bits)    -> Tensor   main.cu:60-91
 
+plus one op the reference does not have, ``gemm_kbit(in, qweight, lut, w_bits)``: the
+fused dequant -> MFMA GEMM for up to ``GEMM_MAX_M`` activation rows (the reference's
+``dequant_kbit`` + ``torch.matmul`` branch, AnyPrecisionLinear.py:60-62, in one launch).
+
 The ops validate their arguments, allocate the result with torch and hand raw
 device pointers plus torch's current HIP stream to libanyprec_hip.so.  Where
 the reference asserts (compiled out in release builds) or exits the process,
@@ -18,7 +22,9 @@ import torch
 
 from any_precision_amd import _capi
 
-__all__ = ["matmul_kbit", "dequant_kbit"]
+__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "GEMM_MAX_M"]
+
+GEMM_MAX_M = _capi.GEMM_MAX_M
 
 _lib = _capi.lib
 
@@ -77,4 +83,27 @@ def matmul_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_b
         rc = _lib.ap_matmul_kbit(in_.data_ptr(), qweight.data_ptr(), lut.data_ptr(), out.data_ptr(), M, N, K,
                                  w_bits, torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "matmul_kbit")
+    return out
+
+
+def gemm_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:
+    """fp16 in_.shape[:-1] + [N] = in_ @ dequant(qweight, lut, w_bits).T for 1 <= M <= GEMM_MAX_M rows,
+    without materialising the fp16 weight."""
+    N, K = _check_weight(qweight, lut, w_bits, "gemm_kbit")
+    if in_.dtype != torch.float16:
+        raise ValueError(f"gemm_kbit: input must be float16, got {in_.dtype}")
+    if in_.device != qweight.device:
+        raise ValueError(f"gemm_kbit: input on {in_.device}, weight on {qweight.device}")
+    if in_.dim() < 1 or in_.shape[-1] != K:
+        raise ValueError(f"gemm_kbit: input last dim must be K={K}, got {tuple(in_.shape)}")
+    M = in_.numel() // K
+    if M < 1 or M > GEMM_MAX_M:
+        raise ValueError(f"gemm_kbit: batch M={M} outside 1..{GEMM_MAX_M}; use dequant_kbit + matmul beyond")
+    if not in_.is_contiguous():
+        raise ValueError("gemm_kbit: input must be contiguous")
+    with torch.cuda.device(qweight.device):
+        out = torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device)
+        rc = _lib.ap_gemm_kbit(in_.data_ptr(), qweight.data_ptr(), lut.data_ptr(), out.data_ptr(), M, N, K,
+                               w_bits, torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "gemm_kbit")
     return out

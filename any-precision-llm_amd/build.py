@@ -47,8 +47,8 @@ def _run(cmd, verbose):
         print(out)
 
 
-def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 7) -> str:
-    """One object per GEMV bit-width (compiled in parallel) + the C ABI, linked into the .so."""
+def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 8) -> str:
+    """One object per kernel family and bit-width (compiled in parallel) + the C ABI, linked into the .so."""
     from concurrent.futures import ThreadPoolExecutor
 
     os.makedirs(OBJDIR, exist_ok=True)
@@ -57,6 +57,7 @@ def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 7) -> str:
     units = [(os.path.join(CSRC, "ap_capi.hip"), os.path.join(OBJDIR, "ap_capi.o"), [])]
     for b in range(3, 9):
         units.append((os.path.join(CSRC, "ap_gemv_inst.hip"), os.path.join(OBJDIR, f"ap_gemv_b{b}.o"), [f"-DAP_BITS={b}"]))
+        units.append((os.path.join(CSRC, "ap_gemm_inst.hip"), os.path.join(OBJDIR, f"ap_gemm_b{b}.o"), [f"-DAP_BITS={b}"]))
     hipcc = _hipcc()
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda u: _run([hipcc, *compile_flags, *u[2], u[0], "-o", u[1]], verbose), units))

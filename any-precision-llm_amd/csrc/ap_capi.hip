@@ -5,6 +5,7 @@
 
 #include "anyprec_hip.h"
 #include "ap_dequant.hpp"
+#include "ap_gemm_launch.hpp"
 #include "ap_gemv_launch.hpp"
 
 namespace {
@@ -18,6 +19,7 @@ struct Tuning {
     int force_rows;    // > 0: rows per wave, overrides target_waves
     int force_wpl;     // > 0: words per lane
     int dequant_blocks_per_cu;
+    int gemm_target_waves;  // waves the fused GEMM grid aims for (K-split follows)
 };
 
 int env_int(const char *name, int dflt) {
@@ -31,6 +33,7 @@ const Tuning &tuning() {
         env_int("AP_GEMV_ROWS", 0),
         env_int("AP_GEMV_WPL", 0),
         env_int("AP_DEQUANT_BLOCKS_PER_CU", 8),
+        env_int("AP_GEMM_TARGET_WAVES", 4096),
     };
     return t;
 }
@@ -132,6 +135,34 @@ int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segm
     if (rows) *rows = geo.R;
     if (grid) *grid = geo.grid;
     return AP_OK;
+}
+
+int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
+                 int w_bits, void *stream) {
+    if (!x || !qweight || !lut || !out) return AP_ENULL;
+    const int rc = check_common(N, K, w_bits);
+    if (rc != AP_OK) return rc;
+    if (M < 1 || M > kGemmMaxM) return AP_EBATCH;
+    if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
+    GemmGeometry geo;
+    geo.mb = (M + 15) / 16;
+    geo.grid = (N + 15) / 16;
+    const int steps = ((K >> 5) + 3) / 4;
+    int ks = (tuning().gemm_target_waves + geo.grid - 1) / geo.grid;
+    if (ks > 8) ks = 8;
+    if (ks > steps) ks = steps;
+    if (ks < 1) ks = 1;
+    geo.ks = ks;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (w_bits) {
+        case 3: launch_gemm<3>(geo, x, qweight, lut, out, M, N, K, st); break;
+        case 4: launch_gemm<4>(geo, x, qweight, lut, out, M, N, K, st); break;
+        case 5: launch_gemm<5>(geo, x, qweight, lut, out, M, N, K, st); break;
+        case 6: launch_gemm<6>(geo, x, qweight, lut, out, M, N, K, st); break;
+        case 7: launch_gemm<7>(geo, x, qweight, lut, out, M, N, K, st); break;
+        default: launch_gemm<8>(geo, x, qweight, lut, out, M, N, K, st); break;
+    }
+    return launch_status();
 }
 
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N,

@@ -53,6 +53,13 @@ int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                    uint16_t *out, int M, int N, int K, int w_bits, void *stream);
 
+/* Fused dequant -> MFMA GEMM, 1 <= M <= 128: out[M,N] = x[M,K] . dequant(qweight, lut)^T
+ * without materialising the fp16 weight.  No single counterpart in the reference: it is the
+ * M > 8 branch of AnyPrecisionLinear.forward (AnyPrecisionLinear.py:60-62: dequant_kbit,
+ * main.cu:60-91, then torch.matmul) in one launch.  fp32 accumulation, fp16 result. */
+int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                 uint16_t *out, int M, int N, int K, int w_bits, void *stream);
+
 /* Human-readable text for a return code of the functions above. */
 const char *ap_strerror(int code);
 

@@ -1,0 +1,125 @@
+"""gemm_kbit (fused dequant -> MFMA GEMM, M up to 128) on the GPU against the oracle,
+through the C ABI.  Tolerance: 1e-2 relative (normwise and against max |y|)."""
+import numpy as np
+import pytest
+import torch
+
+from _util import assert_bit_exact, assert_close_gemv, layer_to_gpu, make
+from any_precision_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+RAGGED = [(1, 32), (7, 32), (5, 96), (13, 1056), (20, 2080), (130, 992), (33, 1024), (17, 3104), (21, 4128)]
+SLICES = [(256, 4096), (176, 11008), (144, 14336)]
+BATCHES = (1, 9, 16, 17, 40, 64, 100, 128)
+
+
+@pytest.fixture(scope="module")
+def ext():
+    import any_precision_ext
+    return any_precision_ext
+
+
+def _x(M, K, seed=0):
+    x = synth.make_x(M, K, seed)
+    return x, torch.from_numpy(x).cuda()
+
+
+@pytest.mark.parametrize("N,K", RAGGED)
+def test_ragged_shapes_all_bits(ext, oracle, N, K):
+    L = make(N, K, seed=N + K)
+    q, luts = layer_to_gpu(L)
+    for b in range(3, 9):
+        for M in (1, 9, 16, 33, 128):
+            print(f"gemm N={N} K={K} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            got = ext.gemm_kbit(xg, q, luts[b], b)
+            assert got.shape == (M, N) and got.dtype == torch.float16
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+
+
+@pytest.mark.parametrize("N,K", SLICES)
+def test_row_slices_of_benchmark_shapes_all_batches(ext, oracle, N, K):
+    L = make(N, K, seed=5)
+    q, luts = layer_to_gpu(L)
+    for b in range(3, 9):
+        for M in BATCHES:
+            print(f"gemm N={N} K={K} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            got = ext.gemm_kbit(xg, q, luts[b], b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+
+
+@pytest.mark.parametrize("N,K", [(4096, 4096), (11008, 4096), (4096, 11008)])
+def test_benchmark_shapes(ext, oracle, N, K):
+    L = make(N, K, seed=1)
+    q, luts = layer_to_gpu(L)
+    for b in (3, 5, 8):
+        for M in (16, 64):
+            print(f"gemm N={N} K={K} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            got = ext.gemm_kbit(xg, q, luts[b], b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+
+
+def test_one_hot_rows_return_dequant_columns_exactly(ext, oracle):
+    # row m of x is e_{k_m}: out[m, :] is column k_m of the dequantised weight, exactly
+    N, K = 48, 3104
+    L = make(N, K, seed=8)
+    q, luts = layer_to_gpu(L)
+    ks = [0, 7, 8, 255, 256, 1023, 1024, 2047, 2048, 3071, 3072, 3080, 3103, 31, 32, 1500, 2999, 100]
+    x = torch.zeros((len(ks), K), dtype=torch.float16, device="cuda")
+    for m, k in enumerate(ks):
+        x[m, k] = 1.0
+    for b in (3, 4, 6, 8):
+        w = oracle.dequant_kbit(L.qweight, L.luts[b], b)
+        got = ext.gemm_kbit(x, q, luts[b], b)
+        for m, k in enumerate(ks):
+            assert_bit_exact(got[m], w[:, k], f"b={b} k={k}")
+
+
+def test_matches_gemv_and_is_deterministic(ext):
+    N, K = 512, 4096
+    L = make(N, K, seed=3)
+    q, luts = layer_to_gpu(L)
+    _, xg = _x(8, K)
+    a = ext.gemm_kbit(xg, q, luts[6], 6)
+    for _ in range(3):
+        assert torch.equal(ext.gemm_kbit(xg, q, luts[6], 6).view(torch.int16), a.view(torch.int16))
+    v = ext.matmul_kbit(xg, q, luts[6], 6).float()
+    assert (a.float() - v).norm() <= 2e-3 * v.norm()
+    y3 = ext.gemm_kbit(xg.reshape(2, 4, K), q, luts[6], 6)
+    assert y3.shape == (2, 4, N) and torch.equal(y3.reshape(8, N).view(torch.int16), a.view(torch.int16))
+
+
+def test_batch_limit_and_errors(ext):
+    L = make(16, 64, seed=0)
+    q, luts = layer_to_gpu(L)
+    with pytest.raises(ValueError, match="1..128"):
+        ext.gemm_kbit(torch.zeros((129, 64), dtype=torch.float16, device="cuda"), q, luts[3], 3)
+    with pytest.raises(ValueError, match="float16"):
+        ext.gemm_kbit(torch.zeros((16, 64), dtype=torch.float32, device="cuda"), q, luts[3], 3)
+
+
+def test_graph_replay_matches_eager(ext):
+    from any_precision_amd import _capi
+    N, K, M = 1024, 4096, 32
+    L = make(N, K, seed=4)
+    q, luts = layer_to_gpu(L)
+    _, xg = _x(M, K)
+    eager = ext.gemm_kbit(xg, q, luts[4], 4)
+    out = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        rc = _capi.lib.ap_gemm_kbit(xg.data_ptr(), q.data_ptr(), luts[4].data_ptr(), out.data_ptr(), M, N, K, 4,
+                                    torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+    for rep in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), rep
