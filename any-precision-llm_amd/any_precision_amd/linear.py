@@ -5,7 +5,7 @@ Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]
 ``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
 ``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
 Batch dispatch: up to 8 activation rows -> ``matmul_kbit`` as in the reference (:60-64);
-9 .. ``GEMM_MAX_M`` rows -> the fused ``gemm_kbit``; beyond -> ``dequant_kbit`` +
+9 .. ``FUSED_GEMM_ROWS`` rows -> the fused ``gemm_kbit``; beyond -> ``dequant_kbit`` +
 ``torch.matmul`` as in the reference.
 """
 from __future__ import annotations
@@ -17,6 +17,12 @@ try:
     from any_precision_ext import matmul_kbit, dequant_kbit, gemm_kbit, GEMM_MAX_M
 except ModuleNotFoundError:
     matmul_kbit, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, 0
+
+
+# Up to this many activation rows the fused GEMM beats dequant_kbit + torch.matmul on every
+# Llama-2-7B shape and bit-width measured (1.3-2.6x at 16 rows); beyond, the re-read of the
+# activations per 16 weight rows costs more than materialising the weight once.
+FUSED_GEMM_ROWS = min(32, GEMM_MAX_M)
 
 
 class AnyPrecisionLinear(nn.Module):
@@ -63,7 +69,7 @@ class AnyPrecisionLinear(nn.Module):
         rows = x.numel() // x.shape[-1]
         if rows <= 8:
             x = matmul_kbit(x, self.qweight, lut, w_bits)
-        elif rows <= GEMM_MAX_M and x.is_contiguous():
+        elif rows <= FUSED_GEMM_ROWS and x.is_contiguous():
             x = gemm_kbit(x, self.qweight, lut, w_bits)      # fused dequant -> MFMA, weight never materialised
         else:
             weight = dequant_kbit(self.qweight, lut, w_bits)
