@@ -147,7 +147,8 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     GemmGeometry geo;
     geo.mb = (M + 15) / 16;
     geo.grid = (N + 15) / 16;
-    const int steps = ((K >> 5) + 3) / 4;
+    const int W = K >> 5;
+    const int steps = (W & 3) == 0 ? (W + 15) / 16 : (W + 3) / 4;  // the kernel's steps along K
     int ks = (tuning().gemm_target_waves + geo.grid - 1) / geo.grid;
     if (ks > 8) ks = 8;
     if (ks > steps) ks = steps;

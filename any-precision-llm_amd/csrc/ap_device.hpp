@@ -56,6 +56,28 @@ __device__ __forceinline__ uint32_t byte_offset(uint32_t v) {
     }
 }
 
+// base + ((v >> 8*BYTE) & 0xff) in one VALU instruction (SDWA byte select on the second
+// addend): the LDS byte address of a gather whose table base differs per lane, for index
+// bytes that already hold the byte offset.
+template <int BYTE>
+__device__ __forceinline__ uint32_t byte_add(uint32_t base, uint32_t v) {
+    static_assert(BYTE >= 0 && BYTE < 4, "");
+    uint32_t r;
+    if constexpr (BYTE == 0)
+        asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0"
+            : "=v"(r) : "v"(base), "v"(v));
+    else if constexpr (BYTE == 1)
+        asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1"
+            : "=v"(r) : "v"(base), "v"(v));
+    else if constexpr (BYTE == 2)
+        asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2"
+            : "=v"(r) : "v"(base), "v"(v));
+    else
+        asm("v_add_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3"
+            : "=v"(r) : "v"(base), "v"(v));
+    return r;
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
     const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);

@@ -14,16 +14,18 @@ void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qwe
     const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
     half_t *oh = reinterpret_cast<half_t *>(out);
     const dim3 block(kWave, geo.ks), grid(geo.grid);
+    const bool vec4 = ((K >> 5) & 3) == 0;  // whole 16-byte quads of words per row
+#define AP_GEMM_CASE(MBV)                                                                                   \
+    case MBV:                                                                                               \
+        if (vec4) gemm_kbit_kernel<BITS, MBV, true><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);  \
+        else gemm_kbit_kernel<BITS, MBV, false><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);      \
+        break;
     switch (geo.mb) {
-        case 1: gemm_kbit_kernel<BITS, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        case 2: gemm_kbit_kernel<BITS, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        case 3: gemm_kbit_kernel<BITS, 3><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        case 4: gemm_kbit_kernel<BITS, 4><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        case 5: gemm_kbit_kernel<BITS, 5><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        case 6: gemm_kbit_kernel<BITS, 6><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        case 7: gemm_kbit_kernel<BITS, 7><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
-        default: gemm_kbit_kernel<BITS, 8><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K); break;
+        AP_GEMM_CASE(1) AP_GEMM_CASE(2) AP_GEMM_CASE(3) AP_GEMM_CASE(4)
+        AP_GEMM_CASE(5) AP_GEMM_CASE(6) AP_GEMM_CASE(7)
+        default: AP_GEMM_CASE(8)
     }
+#undef AP_GEMM_CASE
 }
 
 template void launch_gemm<AP_BITS>(const GemmGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *,
