@@ -20,6 +20,7 @@ struct Tuning {
     int force_wpl;     // > 0: words per lane
     int dequant_blocks_per_cu;
     int gemm_target_waves;  // waves the fused GEMM grid aims for (K-split follows)
+    int mfma_from_rows;     // ap_matmul_kbit uses the MFMA kernel from this many activation rows on
 };
 
 int env_int(const char *name, int dflt) {
@@ -34,6 +35,7 @@ const Tuning &tuning() {
         env_int("AP_GEMV_WPL", 0),
         env_int("AP_DEQUANT_BLOCKS_PER_CU", 8),
         env_int("AP_GEMM_TARGET_WAVES", 4096),
+        env_int("AP_MATMUL_MFMA_FROM", 5),
     };
     return t;
 }
@@ -137,13 +139,13 @@ int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segm
     return AP_OK;
 }
 
-int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
-                 int w_bits, void *stream) {
-    if (!x || !qweight || !lut || !out) return AP_ENULL;
-    const int rc = check_common(N, K, w_bits);
-    if (rc != AP_OK) return rc;
-    if (M < 1 || M > kGemmMaxM) return AP_EBATCH;
-    if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
+}  // extern "C"
+
+namespace {
+
+// Launch of the fused dequant -> MFMA kernel (arguments already checked).
+int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
+             int w_bits, hipStream_t st) {
     GemmGeometry geo;
     geo.mb = (M + 15) / 16;
     geo.grid = (N + 15) / 16;
@@ -154,7 +156,6 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     if (ks > steps) ks = steps;
     if (ks < 1) ks = 1;
     geo.ks = ks;
-    hipStream_t st = static_cast<hipStream_t>(stream);
     switch (w_bits) {
         case 3: launch_gemm<3>(geo, x, qweight, lut, out, M, N, K, st); break;
         case 4: launch_gemm<4>(geo, x, qweight, lut, out, M, N, K, st); break;
@@ -166,6 +167,20 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     return launch_status();
 }
 
+}  // namespace
+
+extern "C" {
+
+int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
+                 int w_bits, void *stream) {
+    if (!x || !qweight || !lut || !out) return AP_ENULL;
+    const int rc = check_common(N, K, w_bits);
+    if (rc != AP_OK) return rc;
+    if (M < 1 || M > kGemmMaxM) return AP_EBATCH;
+    if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
+    return run_gemm(x, qweight, lut, out, M, N, K, w_bits, static_cast<hipStream_t>(stream));
+}
+
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N,
                    int K, int w_bits, void *stream) {
     if (!x || !qweight || !lut || !out) return AP_ENULL;
@@ -174,6 +189,9 @@ int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *l
     if (rc != AP_OK) return rc;
     if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // From 5 activation rows on, the MFMA kernel (cost flat in M up to 16 rows) is faster than
+    // the dot-product kernel (cost linear in M) on most shapes and bit-widths.
+    if (M >= tuning().mfma_from_rows) return run_gemm(x, qweight, lut, out, M, N, K, w_bits, st);
     switch (w_bits) {
         case 3: launch_gemv<3>(M, geo, x, qweight, lut, out, N, K, st); break;
         case 4: launch_gemv<4>(M, geo, x, qweight, lut, out, N, K, st); break;
