@@ -41,6 +41,7 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--table", default="", help="also write the per-layer table (markdown) to this file")
     ap.add_argument("--only-step", action="store_true", help="skip the per-kernel table (used under rocprofv3)")
+    ap.add_argument("--no-extras", action="store_true", help="skip the dequant and batch tables")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies, so a counter run has a kernel of known "
                          "HBM traffic (read 256 MiB, write 256 MiB) to scale FETCH_SIZE / WRITE_SIZE with")
@@ -94,18 +95,39 @@ def main():
         need = int(args.pool_gb * 1e9 / (3 * N * K / 8)) + 1
         sets = max(need, len(idxs) * args.pool)
         pools[(N, K)] = WeightPool(torch, N, K, sets, gen)
-    xs = {K: torch.randn((1, K), device="cuda", generator=gen).to(torch.float16) for K in {K for _, _, K in shapes}}
+    batches = (1, 2, 4, 8, 16, 32)
+    xb = {(M, K): torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+          for K in {K for _, _, K in shapes} for M in batches}
+    for P in pools.values():
+        P.out = torch.empty((max(batches), P.N), dtype=torch.float16, device="cuda")
+    side = torch.cuda.Stream()
     torch.cuda.synchronize()
     cursor = {k: 0 for k in pools}
 
-    def launch(N: int, K: int, b: int, stream: int):
-        """One GEMV on the next weight set of its shape."""
+    def launch(N: int, K: int, b: int, stream: int, M: int = 1, fn=None):
+        """One GEMV (or `fn`: another entry point with the same signature) on the next weight set of its shape."""
         P = pools[(N, K)]
         j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
-        rc = lib.ap_matmul_kbit(xs[K].data_ptr(), P.qweight[j].data_ptr(), P.luts[b][j].data_ptr(),
-                                P.out.data_ptr(), 1, N, K, b, stream)
+        rc = (fn or lib.ap_matmul_kbit)(xb[(M, K)].data_ptr(), P.qweight[j].data_ptr(), P.luts[b][j].data_ptr(),
+                                        P.out.data_ptr(), M, N, K, b, stream)
         if rc != 0:
             raise RuntimeError(_capi.strerror(rc))
+
+    def time_graph(enqueue, reps):
+        """us per call of `enqueue(stream)`: `reps` calls captured in one HIP graph, second replay timed."""
+        with torch.cuda.stream(side):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                for _ in range(reps):
+                    enqueue(torch.cuda.current_stream().cuda_stream)
+            g.replay()
+            side.synchronize()
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record(side)
+            g.replay()
+            a1.record(side)
+            side.synchronize()
+        return a0.elapsed_time(a1) * 1e3 / reps
 
     def step(i: int, stream: int):
         for b in BITS:
@@ -123,7 +145,6 @@ def main():
         del src, dst
 
     # ---- whole-step timing: the K steps are captured in one HIP graph so the host never starves the GPU
-    side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         for i in range(args.warmup):
             step(i, side.cuda_stream)
@@ -152,28 +173,47 @@ def main():
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # ---- per-kernel table: each (shape, w_bits) alone, rotating over the pool (cold planes)
-    table = []
+    table, dequant_table, batch_table = [], [], []
     if not args.only_step:
-        with torch.cuda.stream(side):
-            for (N, K), idxs in uniq.items():
-                for b in BITS:
-                    g = torch.cuda.CUDAGraph()
-                    with torch.cuda.graph(g, stream=side):
-                        for r in range(args.kernel_reps):
-                            launch(N, K, b, torch.cuda.current_stream().cuda_stream)
-                    g.replay()
-                    side.synchronize()
-                    a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    a0.record(side)
-                    g.replay()
-                    a1.record(side)
-                    side.synchronize()
-                    us = a0.elapsed_time(a1) * 1e3 / args.kernel_reps
-                    by = synth.gemv_bytes(N, K, b, 1)
-                    geo = _capi.matmul_geometry(1, N, K, b)
-                    table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 3), "GBps": round(by / us / 1e3, 1),
-                                  "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": by,
-                                  "count_in_step": len(idxs), "geometry": geo})
+        for (N, K), idxs in uniq.items():
+            for b in BITS:
+                us = time_graph(lambda st: launch(N, K, b, st), args.kernel_reps)
+                by = synth.gemv_bytes(N, K, b, 1)
+                geo = _capi.matmul_geometry(1, N, K, b)
+                table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 3), "GBps": round(by / us / 1e3, 1),
+                              "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": by,
+                              "count_in_step": len(idxs), "geometry": geo})
+
+    # ---- further kernels of the path (reported beside the headline, not part of `value`)
+    if not args.only_step and not args.no_extras:
+        # dequant_kbit: planes + table in, fp16 [N, K] out; outputs rotate over >= 512 MB of buffers
+        for (N, K), P in pools.items():
+            nout = max(2, int(512e6 / (2 * N * K)) + 1)
+            outs = [torch.empty((N, K), dtype=torch.float16, device="cuda") for _ in range(nout)]
+            state = {"i": 0}
+
+            def deq(st, b):
+                j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
+                state["i"] = (state["i"] + 1) % nout
+                rc = lib.ap_dequant_kbit(P.qweight[j].data_ptr(), P.luts[b][j].data_ptr(),
+                                         outs[state["i"]].data_ptr(), N, K, b, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+
+            for b in BITS:
+                us = time_graph(lambda st: deq(st, b), 12)
+                by = synth.dequant_bytes(N, K, b)
+                dequant_table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 2),
+                                      "GBps": round(by / us / 1e3, 1), "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4)})
+            del outs
+        # batches: matmul_kbit for M <= 8 (MFMA kernel from 5 rows on), fused gemm_kbit for 16 and 32 rows
+        for (N, K) in pools:
+            for b in (3, 4, 8):
+                row = {"N": N, "K": K, "w_bits": b}
+                for M in batches:
+                    fn = lib.ap_matmul_kbit if M <= 8 else lib.ap_gemm_kbit
+                    row[f"us_M{M}"] = round(time_graph(lambda st: launch(N, K, b, st, M, fn), 24), 2)
+                batch_table.append(row)
 
     roofline = None
     if table:
@@ -225,12 +265,24 @@ def main():
                    "bytes_per_step": step_bytes,
                    "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline, "cpu_baseline": cpu, "layers": table,
+        "dequant_kbit": dequant_table, "batch_us": batch_table,
     }
     if args.table and table:
         with open(args.table, "w") as f:
+            f.write("GEMV batch 1 (matmul_kbit)\n\n")
             f.write("| N x K | w_bits | us/launch | GB/s | % of 8 TB/s |\n|---|---|---|---|---|\n")
             for r in table:
                 f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | {r['us']:.2f} | {r['GBps']:.0f} | {100 * r['frac']:.1f} |\n")
+            if dequant_table:
+                f.write("\ndequant_kbit (read planes + table, write fp16)\n\n")
+                f.write("| N x K | w_bits | us/launch | GB/s | % of 8 TB/s |\n|---|---|---|---|---|\n")
+                for r in dequant_table:
+                    f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | {r['us']:.1f} | {r['GBps']:.0f} | {100 * r['frac']:.1f} |\n")
+            if batch_table:
+                f.write("\nus per launch by batch (M <= 8: matmul_kbit; 16, 32: gemm_kbit)\n\n")
+                f.write("| N x K | w_bits | " + " | ".join(f"M={M}" for M in batches) + " |\n|---|---|" + "---|" * len(batches) + "\n")
+                for r in batch_table:
+                    f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | " + " | ".join(f"{r[f'us_M{M}']:.1f}" for M in batches) + " |\n")
     print(json.dumps(result))
 
 
