@@ -33,7 +33,7 @@ const Tuning &tuning() {
         env_int("AP_GEMV_TARGET_WAVES", 16384),
         env_int("AP_GEMV_ROWS", 0),
         env_int("AP_GEMV_WPL", 0),
-        env_int("AP_DEQUANT_BLOCKS_PER_CU", 8),
+        env_int("AP_DEQUANT_BLOCKS_PER_CU", 32),
         env_int("AP_GEMM_TARGET_WAVES", 4096),
         env_int("AP_MATMUL_MFMA_FROM", 5),
     };
@@ -77,10 +77,11 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
 
 template <int BITS>
 void launch_dequant(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream) {
-    int blocks = (N + kDequantWaves - 1) / kDequantWaves;
-    const int cap = kNumCUs * tuning().dequant_blocks_per_cu;
+    const int S = ((K >> 5) + kWave - 1) / kWave;  // 64-word segments per row
+    long long blocks = ((long long)N * S + kDequantWaves - 1) / kDequantWaves;
+    const long long cap = (long long)kNumCUs * tuning().dequant_blocks_per_cu;
     if (blocks > cap) blocks = cap;
-    dequant_kbit_kernel<BITS><<<dim3(blocks), dim3(kDequantWaves * kWave), 0, stream>>>(
+    dequant_kbit_kernel<BITS><<<dim3((unsigned)blocks), dim3(kDequantWaves * kWave), 0, stream>>>(
         qweight, reinterpret_cast<const half_t *>(lut), reinterpret_cast<half_t *>(out), N, K);
 }
 

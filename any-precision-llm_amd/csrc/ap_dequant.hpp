@@ -4,11 +4,13 @@
 // (any_precision/modules/kernels/dequant.cuh:177-242).  Result is a pure
 // table copy, hence bit-exact by construction when the index is right.
 //
-// Mapping: one wave64 per row at a time; lane l owns word l, l+64, ... of the
-// row.  Per word a lane reads one dword per plane (a wave covers 256 B of each
-// plane, fully coalesced), rebuilds its 32 indices in registers, gathers from
-// the row's table in LDS and emits four 16-byte stores; for a fixed byte
-// group the 32 lanes of a chunk write 512 contiguous bytes.
+// Mapping: the unit of work is one 64-word segment of one row (2048 elements); a wave
+// takes segments in a grid-stride loop, lane l owns word l of the segment.  Per word a
+// lane reads one dword per plane (a wave covers 256 B of each plane, fully coalesced),
+// rebuilds its 32 indices in registers, gathers from the row's table in LDS and emits four
+// 16-byte stores; for a fixed byte group the 32 lanes of a chunk write 512 contiguous
+// bytes.  Cutting rows into segments keeps the number of independent waves proportional to
+// the bytes, whatever the row length.
 #pragma once
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
@@ -27,20 +29,24 @@ __global__ __launch_bounds__(kDequantWaves * kWave) void dequant_kbit_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int W = K >> 5;
-    const int wave_stride = gridDim.x * kDequantWaves;
+    const int S = (W + kWave - 1) / kWave;  // segments per row
+    const long long items = (long long)N * S;
+    const long long stride = (long long)gridDim.x * kDequantWaves;
     const size_t plane_stride = (size_t)N * W;
 
     int buf = 0;
-    for (int row = blockIdx.x * kDequantWaves + wave; row < N; row += wave_stride, buf ^= 1) {
+    for (long long item = (long long)blockIdx.x * kDequantWaves + wave; item < items; item += stride, buf ^= 1) {
+        const int row = (int)(item / S), seg = (int)(item - (long long)row * S);
         half_t *tab = tables[wave][buf];
         lut_stage<BITS>(lut_fetch<BITS>(lut + (size_t)row * NC, lane), tab, lane);
         // LDS operations of one wave complete in order, so the table is
         // visible to the gathers below without a workgroup barrier.
         __builtin_amdgcn_wave_barrier();
 
-        const uint32_t *wrow = qweight + (size_t)row * W;
-        half_t *orow = out + (size_t)row * K;
-        for (int w = lane; w < W; w += kWave) {
+        const int w = seg * kWave + lane;
+        if (w < W) {
+            const uint32_t *wrow = qweight + (size_t)row * W;
+            half_t *orow = out + (size_t)row * K;
             uint32_t q[BITS];
 #pragma unroll
             for (int p = 0; p < BITS; p++) q[p] = __builtin_nontemporal_load(wrow + p * plane_stride + w);
