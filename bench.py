@@ -114,8 +114,19 @@ def main():
             raise RuntimeError(_capi.strerror(rc))
 
     def time_graph(enqueue, reps):
-        """us per call of `enqueue(stream)`: `reps` calls captured in one HIP graph, second replay timed."""
+        """us per call of `enqueue(stream)`: `reps` calls captured in one HIP graph, second replay timed
+        (with --eager: launched one by one, host launch cost included)."""
         with torch.cuda.stream(side):
+            if args.eager:
+                enqueue(side.cuda_stream)
+                side.synchronize()
+                a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a0.record(side)
+                for _ in range(reps):
+                    enqueue(side.cuda_stream)
+                a1.record(side)
+                side.synchronize()
+                return a0.elapsed_time(a1) * 1e3 / reps
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=side):
                 for _ in range(reps):
