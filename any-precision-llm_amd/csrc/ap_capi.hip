@@ -19,8 +19,8 @@ struct Tuning {
     int force_rows;    // > 0: rows per wave, overrides target_waves
     int force_wpl;     // > 0: words per lane
     int dequant_blocks_per_cu;
-    int gemm_target_waves;  // waves the fused GEMM grid aims for (K-split follows)
     int mfma_from_rows;     // ap_matmul_kbit uses the MFMA kernel from this many activation rows on
+    int force_gemm_split;   // > 0: K-split waves per workgroup of the fused GEMM
 };
 
 int env_int(const char *name, int dflt) {
@@ -34,8 +34,8 @@ const Tuning &tuning() {
         env_int("AP_GEMV_ROWS", 0),
         env_int("AP_GEMV_WPL", 0),
         env_int("AP_DEQUANT_BLOCKS_PER_CU", 32),
-        env_int("AP_GEMM_TARGET_WAVES", 4096),
         env_int("AP_MATMUL_MFMA_FROM", 5),
+        env_int("AP_GEMM_SPLIT", 0),
     };
     return t;
 }
@@ -152,8 +152,10 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     geo.grid = (N + 15) / 16;
     const int W = K >> 5;
     const int steps = (W & 3) == 0 ? (W + 15) / 16 : (W + 3) / 4;  // the kernel's steps along K
-    int ks = (tuning().gemm_target_waves + geo.grid - 1) / geo.grid;
-    if (ks > 8) ks = 8;
+    // As many K-split waves as a workgroup holds: every split measured slower with fewer
+    // (the grid alone, N/16 workgroups, is far too small to fill 256 CUs).
+    int ks = tuning().force_gemm_split > 0 ? tuning().force_gemm_split : kGemmMaxSplit;
+    if (ks > kGemmMaxSplit) ks = kGemmMaxSplit;
     if (ks > steps) ks = steps;
     if (ks < 1) ks = 1;
     geo.ks = ks;

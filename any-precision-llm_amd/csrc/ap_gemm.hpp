@@ -28,16 +28,19 @@
 // VEC4 a lane loads one word per step (16 contiguous bytes per row and instruction) and
 // the 64-byte line is re-read from L1/L2 by the next three steps.
 #pragma once
+#include <type_traits>
+
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
+#include "ap_gemm_launch.hpp"
 
 namespace ap {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kGemmRows = 16;     // weight rows per workgroup (one MFMA column block)
-constexpr int kGemmMaxSplit = 8;  // K-split waves per workgroup
 
 // 4x4 transpose of r[0..3] across the four 16-lane rows of the wave: on return r[i] of
 // row g holds what r[g] of row i held.
@@ -58,7 +61,8 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K) {
     constexpr int NC = 1 << BITS;
-    constexpr int WPS = VEC4 ? 4 : 1;  // words per lane and step
+    constexpr int WPS = VEC4 ? 4 : 1;             // words per lane and step
+    constexpr int TQ = kGemmRows * NC / 8;  // 16-byte quads of the 16 tables
     __shared__ __attribute__((aligned(16))) half_t tables[kGemmRows][NC];
     __shared__ float red[kGemmMaxSplit][MB][4][kWave];
 
@@ -70,28 +74,9 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const int n0 = blockIdx.x * kGemmRows;
     const int row = min(n0 + col, N - 1);  // rows past N repeat row N-1 and are not stored
 
-    // stage the 16 tables (16 * NC halves) with the whole workgroup
-    {
-        const int nthr = KS * kWave, tid = ks * kWave + lane;
-        const uint32_t *src = reinterpret_cast<const uint32_t *>(lut);
-        uint32_t *dst = reinterpret_cast<uint32_t *>(&tables[0][0]);
-        for (int i = tid; i < kGemmRows * NC / 2; i += nthr) {
-            const int r = i / (NC / 2), c = i - r * (NC / 2);
-            dst[i] = src[(size_t)min(n0 + r, N - 1) * (NC / 2) + c];
-        }
-    }
-    __syncthreads();
-    // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
-    typedef __attribute__((address_space(3))) half_t lds_half_t;
-    const uint32_t tab_base = (uint32_t)(uintptr_t)((lds_half_t *)&tables[0][0]) + (uint32_t)col * (NC * 2);
-
     // this wave's range of steps (4 * WPS words of every row per step)
     const int steps = (W + 4 * WPS - 1) / (4 * WPS);
-    const int s_begin = (int)((long long)steps * ks / KS), s_end = (int)((long long)steps * (ks + 1) / KS);
-
-    float4_t acc[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) acc[mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    const int s_begin = steps * ks / KS, s_end = steps * (ks + 1) / KS;  // steps <= 512
 
     const uint32_t *wrow = qweight + (size_t)row * W;
     // q[p][i]: plane p, i-th word of this lane for the step
@@ -114,61 +99,127 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
         }
     };
 
+    // Load order: planes of the first step, then the tables -- both are in flight together
+    // and the tables are staged while nothing else could run anyway.  The 16 tables are
+    // contiguous in lut (rows past N re-read the last 16 bytes of the array; their columns
+    // are never stored).
     uint32_t qn[BITS][WPS];
     if (s_begin < s_end) fetch(s_begin, qn);
-    for (int step = s_begin; step < s_end; step++) {
-        uint32_t q[BITS][WPS];
+    {
+        const int nthr = KS * kWave;
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[0][0]);
+        const long long first = (long long)n0 * (NC / 8), last = (long long)N * (NC / 8) - 1;
+        for (int i = ks * kWave + lane; i < TQ; i += nthr) dst[i] = src[min(first + i, last)];
+    }
+    __syncthreads();
+    // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
+    typedef __attribute__((address_space(3))) half_t lds_half_t;
+    const uint32_t tab_base = (uint32_t)(uintptr_t)((lds_half_t *)&tables[0][0]) + (uint32_t)col * (NC * 2);
+
+    // byte offset of this lane's activation row in each row block (rows past M repeat row M-1)
+    uint32_t xoff[MB];
 #pragma unroll
-        for (int p = 0; p < BITS; p++)
+    for (int mb = 0; mb < MB; mb++) xoff[mb] = (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)K * 2u;
+    const int full_chunks = W >> 5;                // chunks of 32 words; a shorter one may follow
+    const uint32_t tail_stride = (uint32_t)(W & 31) * 16u;  // bytes of x between byte groups in the tail chunk
+
+    float4_t acc[MB];
 #pragma unroll
-            for (int i = 0; i < WPS; i++) q[p][i] = qn[p][i];
-        if (step + 1 < s_end) fetch(step + 1, qn);
+    for (int mb = 0; mb < MB; mb++) acc[mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // One step: transpose the planes of each word to indices, gather, multiply.  CHECK: the
+    // step may reach past the end of the row (only the last step of a row can).
+    //
+    // The unit of the inner schedule is the octet (one byte group of one word: one B operand,
+    // MB MFMAs).  The activations of an octet come from L2 and nothing else in the wave can
+    // hide that latency, so they are requested AHEAD octets before they are used.
+    constexpr int OCT = 4 * WPS;
+    constexpr int AHEAD = MB == 1 ? 4 : (MB == 2 ? 2 : 1);
+    auto process = [&](auto check_c, int step, uint32_t(&q)[BITS][WPS]) {
+        constexpr bool CHECK = decltype(check_c)::value;
+        // x byte offset of byte group 0 of each word, and the distance between byte groups
+        uint32_t kb[WPS], jstride[WPS];
+        bool live[WPS];
+#pragma unroll
+        for (int wi = 0; wi < WPS; wi++) {
+            const int w = 4 * (WPS * step + wi) + grp;
+            live[wi] = !CHECK || w < W;  // words past the row end contribute zeros
+            const int wc = live[wi] ? w : W - 1;
+            const int chunk = wc >> 5;
+            kb[wi] = ((uint32_t)chunk << 11) + ((uint32_t)(wc & 31) << 4);
+            jstride[wi] = chunk == full_chunks ? tail_stride : 512u;
+        }
+        half8_t a[OCT][MB];
+        auto load_a = [&](auto t_c) {
+            constexpr int t = decltype(t_c)::value;
+            if constexpr (t < OCT) {
+                const uint32_t koff = kb[t / 4] + (uint32_t)(t % 4) * jstride[t / 4];
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+                    a[t][mb] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(x) + (size_t)(xoff[mb] + koff));
+            }
+        };
+        static_for<AHEAD>([&](auto t_c) { load_a(t_c); });
         if constexpr (VEC4) {
 #pragma unroll
             for (int p = 0; p < BITS; p++) transpose_rows4(q[p]);
         }
-
-        static_for<WPS>([&](auto i_c) {
-            constexpr int wi = decltype(i_c)::value;
-            const int w = 4 * (WPS * step + wi) + grp;
-            const bool live = w < W;  // words past the row end contribute zeros
-            const int wc = live ? w : W - 1;
-
-            uint32_t qq[BITS];
+        // index bytes hold the byte offset into the table (index * 2) where that fits a byte
+        constexpr int PRE = BITS <= 7 ? 1 : 0;
+        uint32_t idx[8];
+        static_for<OCT>([&](auto t_c) {
+            constexpr int t = decltype(t_c)::value, wi = t / 4, j = t % 4, c = 3 - j;
+            load_a(std::integral_constant<int, t + AHEAD>{});
+            if constexpr (j == 0) {
+                uint32_t qq[BITS];
 #pragma unroll
-            for (int p = 0; p < BITS; p++) qq[p] = q[p][wi];
-            // index bytes hold the byte offset into the table (index * 2) where that fits a byte
-            constexpr int PRE = BITS <= 7 ? 1 : 0;
-            uint32_t idx[8];
-            planes_to_indices<BITS, PRE>(qq, idx);
-            static_for<4>([&](auto j_c) {
-                constexpr int j = decltype(j_c)::value, c = 3 - j;
-                // B operand: the eight weights of byte group j
-                u32x4 bw;
-                static_for<4>([&](auto e_c) {
-                    constexpr int i = decltype(e_c)::value;
-                    uint32_t a0, a1;
-                    if constexpr (PRE) {
-                        a0 = byte_add<c>(tab_base, idx[2 * i]);
-                        a1 = byte_add<c>(tab_base, idx[2 * i + 1]);
-                    } else {
-                        a0 = tab_base + byte_offset<c, 1>(idx[2 * i]);
-                        a1 = tab_base + byte_offset<c, 1>(idx[2 * i + 1]);
-                    }
-                    const uint32_t lo = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a0);
-                    const uint32_t hi = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a1);
-                    bw[i] = live ? (lo | (hi << 16)) : 0u;
-                });
-                const half8_t bfrag = __builtin_bit_cast(half8_t, bw);
-                const int k0 = group_base(wc, j, K);
-#pragma unroll
-                for (int mb = 0; mb < MB; mb++) {
-                    const int m = min(mb * 16 + col, M - 1);  // rows past M repeat row M-1 and are not stored
-                    const half8_t afrag = *reinterpret_cast<const half8_t *>(x + (size_t)m * K + k0);
-                    acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag, acc[mb], 0, 0, 0);
+                for (int p = 0; p < BITS; p++) qq[p] = q[p][wi];
+                planes_to_indices<BITS, PRE>(qq, idx);
+            }
+            // B operand: the eight weights of byte group j
+            u32x4 bw;
+            static_for<4>([&](auto e_c) {
+                constexpr int i = decltype(e_c)::value;
+                uint32_t a0, a1;
+                if constexpr (PRE) {
+                    a0 = byte_add<c>(tab_base, idx[2 * i]);
+                    a1 = byte_add<c>(tab_base, idx[2 * i + 1]);
+                } else {
+                    a0 = tab_base + byte_offset<c, 1>(idx[2 * i]);
+                    a1 = tab_base + byte_offset<c, 1>(idx[2 * i + 1]);
                 }
+                half2_t h;
+                h.x = *reinterpret_cast<const lds_half_t *>(a0);
+                h.y = *reinterpret_cast<const lds_half_t *>(a1);
+                const uint32_t packed = __builtin_bit_cast(uint32_t, h);
+                bw[i] = live[wi] ? packed : 0u;
             });
+            const half8_t bfrag = __builtin_bit_cast(half8_t, bw);
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][mb], bfrag, acc[mb], 0, 0, 0);
         });
+    };
+
+    // With few planes the next step's words are fetched while this step computes; with
+    // many, the second register set is not worth its registers (no measurable gain).
+    constexpr bool PREFETCH = BITS * WPS <= 20;
+    for (int step = s_begin; step < s_end; step++) {
+        uint32_t q[BITS][WPS];
+        if (PREFETCH || step == s_begin) {
+#pragma unroll
+            for (int p = 0; p < BITS; p++)
+#pragma unroll
+                for (int i = 0; i < WPS; i++) q[p][i] = qn[p][i];
+        } else {
+            fetch(step, q);
+        }
+        if (PREFETCH && step + 1 < s_end) fetch(step + 1, qn);
+        if (4 * WPS * (step + 1) <= W)
+            process(std::false_type{}, step, q);
+        else
+            process(std::true_type{}, step, q);
     }
 
     // Combine the K-split partial tiles in wave order (also with one wave: it keeps the

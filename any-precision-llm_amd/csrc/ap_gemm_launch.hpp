@@ -6,7 +6,8 @@
 
 namespace ap {
 
-constexpr int kGemmMaxM = 128;  // activation rows one launch serves (8 MFMA row blocks)
+constexpr int kGemmMaxM = 128;    // activation rows one launch serves (8 MFMA row blocks)
+constexpr int kGemmMaxSplit = 8;  // K-split waves per workgroup
 
 struct GemmGeometry {
     int mb;    // activation row blocks of 16
