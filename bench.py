@@ -32,6 +32,11 @@ BITS = (3, 4, 5, 6, 7, 8)
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--workload", default="llama2_7b_layer_batch1",
+                    choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model"),
+                    help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
+                         "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
+                         "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -79,6 +84,10 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.workload == "llama3_8b_layer_batches":
+        return batch_sweep(args, torch, _capi, synth)
+    if args.workload == "llama2_7b_dequant_full_model":
+        return dequant_full_model(args, torch, _capi, synth)
     lib = _capi.lib
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
@@ -295,6 +304,120 @@ def main():
                 for r in batch_table:
                     f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | " + " | ".join(f"{r[f'us_M{M}']:.1f}" for M in batches) + " |\n")
     print(json.dumps(result))
+
+
+def _graph_us(torch, side, enqueue, reps):
+    """us per call of `enqueue(stream)`: `reps` calls in one HIP graph, best of three timed replays."""
+    with torch.cuda.stream(side):
+        enqueue(side.cuda_stream)
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for _ in range(reps):
+                enqueue(torch.cuda.current_stream().cuda_stream)
+        g.replay()
+        side.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a0.record(side)
+            g.replay()
+            a1.record(side)
+            side.synchronize()
+            best = min(best, a0.elapsed_time(a1) * 1e3 / reps)
+    return best
+
+
+def batch_sweep(args, torch, _capi, synth):
+    """matmul_kbit on the Llama-3-8B linear shapes at M = 1, 2, 4, 8, every w_bits, cold planes."""
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    side = torch.cuda.Stream()
+    rows = []
+    for N, K in sorted({(N, K) for _, N, K in synth.LLAMA3_8B_LAYER}):
+        sets = int(args.pool_gb * 1e9 / (3 * N * K / 8)) + 1
+        P = WeightPool(torch, N, K, sets, gen)
+        cur = {"j": 0}
+        for M in (1, 2, 4, 8):
+            x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+            for b in BITS:
+                def call(st):
+                    cur["j"] = (cur["j"] + 1) % P.sets
+                    rc = lib.ap_matmul_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                            P.out.data_ptr(), M, N, K, b, st)
+                    if rc != 0:
+                        raise RuntimeError(_capi.strerror(rc))
+                us = _graph_us(torch, side, call, min(args.kernel_reps, P.sets))
+                by = synth.gemv_bytes(N, K, b, M)
+                rows.append({"N": N, "K": K, "M": M, "w_bits": b, "us": round(us, 2), "GBps": round(by / us / 1e3, 1),
+                             "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del P
+        torch.cuda.empty_cache()
+    if args.table:
+        with open(args.table, "w") as f:
+            f.write("matmul_kbit, Llama-3-8B linear shapes: us per launch (GB/s of algorithmic bytes)\n\n")
+            f.write("| N x K | M | " + " | ".join(f"b={b}" for b in BITS) + " |\n|---|---|" + "---|" * len(BITS) + "\n")
+            for (N, K, M) in sorted({(r["N"], r["K"], r["M"]) for r in rows}):
+                cells = [next(r for r in rows if (r["N"], r["K"], r["M"], r["w_bits"]) == (N, K, M, b)) for b in BITS]
+                f.write(f"| {N}x{K} | {M} | " + " | ".join(f"{c['us']:.1f} ({c['GBps']:.0f})" for c in cells) + " |\n")
+    # one figure for the sweep: bytes over time of one pass over a layer (7 linears) at every M and w_bits
+    tot_b = tot_t = 0.0
+    for _, N, K in synth.LLAMA3_8B_LAYER:
+        for r in rows:
+            if (r["N"], r["K"]) == (N, K):
+                tot_b += synth.gemv_bytes(N, K, r["w_bits"], r["M"])
+                tot_t += r["us"]
+    print(json.dumps({
+        "metric": "bitplane GEMV effective HBM GB/s, Llama-3-8B layer set, w_bits 3-8, batches 1,2,4,8",
+        "value": round(tot_b / tot_t / 1e3, 1), "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
+        "vs_baseline": None, "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B decoder-layer linear set (q,o 4096x4096; k,v 1024x4096; gate,up 14336x4096; "
+                               "down 4096x14336), M in 1,2,4,8, parent 8 bits, w_bits 3..8; per-kernel graphs of "
+                               f"{args.kernel_reps} launches over cold weight sets"},
+        "kernels": rows}))
+
+
+def dequant_full_model(args, torch, _capi, synth):
+    """dequant_kbit over every linear of a Llama-2-7B-shaped model (32 layers x 7 linears, 6.476 G weights)."""
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    side = torch.cuda.Stream()
+    layers = 32
+    linears = []   # (N, K, qweight [8,N,W], luts {b: [N, 2^b]})
+    for li in range(layers):
+        for _, N, K in synth.LLAMA2_7B_LAYER:
+            q = torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda", generator=gen)
+            luts = {b: torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02, dim=1).values
+                    .to(torch.float16).contiguous() for b in BITS}
+            linears.append((N, K, q, luts))
+    # outputs rotate over ~1 GB of buffers per shape so that no store lands on a line still in the last-level cache
+    outs = {}
+    for N, K in {(N, K) for N, K, _, _ in linears}:
+        outs[(N, K)] = [torch.empty((N, K), dtype=torch.float16, device="cuda") for _ in range(int(1e9 / (2 * N * K)) + 1)]
+    turn = {k: 0 for k in outs}
+    weights = sum(N * K for N, K, _, _ in linears)
+    results = []
+    for b in BITS:
+        def pass_(st):
+            for N, K, q, luts in linears:
+                turn[(N, K)] = (turn[(N, K)] + 1) % len(outs[(N, K)])
+                rc = lib.ap_dequant_kbit(q.data_ptr(), luts[b].data_ptr(), outs[(N, K)][turn[(N, K)]].data_ptr(), N, K, b, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+        us = _graph_us(torch, side, pass_, 1)
+        by = sum(synth.dequant_bytes(N, K, b) for N, K, _, _ in linears)
+        results.append({"w_bits": b, "ms": round(us / 1e3, 3), "GBps": round(by / us / 1e3, 1),
+                        "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": by})
+    tot_b, tot_t = sum(r["bytes"] for r in results), sum(r["ms"] for r in results)
+    print(json.dumps({
+        "metric": "dequant_kbit effective HBM GB/s (read planes + table, write fp16), Llama-2-7B full model, w_bits 3-8",
+        "value": round(tot_b / tot_t / 1e6, 1), "unit": "GB/s", "n_gpus": 1, "higher_is_better": True,
+        "vs_baseline": None, "dtype": "fp16 tables, u32 bitplanes (table copy, bit-exact)", "data": "synthetic",
+        "config": {"workload": f"dequant_kbit over 32 layers x 7 linears = {weights} weights, one HIP graph of 224 "
+                               "launches per w_bits, best of three replays"},
+        "per_w_bits": results}))
 
 
 if __name__ == "__main__":
