@@ -33,10 +33,13 @@ def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--workload", default="llama2_7b_layer_batch1",
-                    choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model"),
+                    choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model",
+                             "llama2_7b_decode"),
                     help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
                          "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
-                         "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.")
+                         "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.  "
+                         "llama2_7b_decode: batch-1 greedy decoding of a random-init Llama-2-7B-shaped model, "
+                         "256 tokens after a 128-token prompt, per w_bits.")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -88,6 +91,9 @@ def main():
         return batch_sweep(args, torch, _capi, synth)
     if args.workload == "llama2_7b_dequant_full_model":
         return dequant_full_model(args, torch, _capi, synth)
+    if args.workload == "llama2_7b_decode":
+        with torch.inference_mode():     # the decoder captures its graphs in inference mode; stay in it
+            return decode_tokens(args, torch, _capi, synth)
     lib = _capi.lib
     gen = torch.Generator(device="cuda")
     gen.manual_seed(0)
@@ -418,6 +424,69 @@ def dequant_full_model(args, torch, _capi, synth):
         "config": {"workload": f"dequant_kbit over 32 layers x 7 linears = {weights} weights, one HIP graph of 224 "
                                "launches per w_bits, best of three replays"},
         "per_w_bits": results}))
+
+
+
+def decode_tokens(args, torch, _capi, synth):
+    """Batch-1 greedy decoding, random-init Llama-2-7B-shaped model: tokens/s per w_bits, the decode
+    step replayed from a HIP graph; beside it the 224 GEMVs of a token alone and the eager loop."""
+    from transformers import LlamaConfig
+    from any_precision_amd import AnyPrecisionForCausalLM, GraphDecoder
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
+                      num_key_value_heads=32, vocab_size=32000, max_position_embeddings=4096, rms_norm_eps=1e-5,
+                      tie_word_embeddings=False)
+    model = AnyPrecisionForCausalLM.from_config(cfg, seed=0, device="cuda")
+    prompt_len, new_tokens = 128, 256
+    dec = GraphDecoder(model, max_len=prompt_len + new_tokens + 8)
+    ids = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=torch.Generator().manual_seed(0)).cuda()
+    lib = _capi.lib
+    side = torch.cuda.Stream()
+    rows = []
+    for b in BITS:
+        dec.prefill(ids, b)
+        dec.capture(b)
+        dec.decode(8, b)                                   # warm replays
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.decode(new_tokens - 9, b)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        tok_s = (new_tokens - 9) / dt
+        eager = None
+        if b in (3, 8):
+            dec.prefill(ids, b)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dec.decode(32, b, use_graph=False)
+            torch.cuda.synchronize()
+            eager = 32 / (time.perf_counter() - t0)
+        # the linears of one token alone (224 GEMVs on this model's own weights, one graph)
+        x = {K: torch.randn((1, K), device="cuda").half() for K in (4096, 11008)}
+        outs = {N: torch.empty((1, N), dtype=torch.float16, device="cuda") for N in (4096, 11008)}
+
+        def token_linears(st):
+            for lin in model.ap_linears:
+                rc = lib.ap_matmul_kbit(x[lin.in_features].data_ptr(), lin.qweight.data_ptr(),
+                                        lin._buffers[f"lut{b}"].data_ptr(), outs[lin.out_features].data_ptr(),
+                                        1, lin.out_features, lin.in_features, b, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+        lin_us = _graph_us(torch, side, token_linears, 1)
+        lin_bytes = sum(synth.gemv_bytes(l.out_features, l.in_features, b, 1) for l in model.ap_linears)
+        rows.append({"w_bits": b, "tokens_per_s": round(tok_s, 1), "ms_per_token": round(1e3 / tok_s, 3),
+                     "eager_tokens_per_s": None if eager is None else round(eager, 1),
+                     "linears_ms_per_token": round(lin_us / 1e3, 3),
+                     "linears_GBps": round(lin_bytes / lin_us / 1e3, 1),
+                     "linears_frac_of_hbm_peak": round(lin_bytes / lin_us / 1e3 / HBM_PEAK_GBS, 4)})
+    print(json.dumps({
+        "metric": "batch-1 decode tokens/s, random-init Llama-2-7B-shaped model, mean over w_bits 3-8",
+        "value": round(sum(r["tokens_per_s"] for r in rows) / len(rows), 1), "unit": "tokens/s", "n_gpus": 1,
+        "higher_is_better": True, "vs_baseline": None, "dtype": "fp16 (fp32 accumulate), u32 bitplanes",
+        "data": "synthetic (random-init weights, random prompt ids)",
+        "config": {"workload": f"greedy decode of {new_tokens} tokens after a {prompt_len}-token prompt, batch 1, "
+                               "32 layers / hidden 4096 / FFN 11008 / 32 heads / vocab 32000; decode step replayed "
+                               "from one HIP graph; linears = this library, everything else stock PyTorch ops"},
+        "per_w_bits": rows}))
 
 
 if __name__ == "__main__":
