@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libanyprec_hip.so")
 
 AP_OK = 0
 AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT = -1, -2, -3, -4, -5, -6
-AP_ABI_VERSION = 1
+AP_ABI_VERSION = 2
 
 if not os.path.exists(LIB_PATH):
     raise ModuleNotFoundError(
@@ -34,6 +34,9 @@ lib.ap_matmul_kbit.restype = _ci
 lib.ap_gemm_kbit.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 lib.ap_gemm_kbit.restype = _ci
 _pi = ctypes.POINTER(ctypes.c_int)
+_pvp = ctypes.POINTER(ctypes.c_void_p)
+lib.ap_matmul_kbit_group.argtypes = [_vp, _ci, _pvp, _pvp, _pvp, _pi, _ci, _ci, _ci, _vp]
+lib.ap_matmul_kbit_group.restype = _ci
 lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi]
 lib.ap_matmul_kbit_geometry.restype = _ci
 
@@ -42,9 +45,18 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
         f"{LIB_PATH} has ABI version {lib.ap_abi_version()}, this binding needs {AP_ABI_VERSION}: rebuild it"
     )
 
-EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_gemm_kbit",
-           "ap_matmul_kbit_geometry")
+EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
+           "ap_gemm_kbit", "ap_matmul_kbit_geometry")
 GEMM_MAX_M = 128
+GROUP_MAX = 4
+
+
+def matmul_group(x_ptr: int, qweights, luts, outs, rows, M: int, K: int, w_bits: int, stream: int) -> int:
+    """ap_matmul_kbit_group on raw device addresses (lists of equal length <= GROUP_MAX)."""
+    n = len(qweights)
+    arr = ctypes.c_void_p * n
+    return lib.ap_matmul_kbit_group(x_ptr, n, arr(*qweights), arr(*luts), arr(*outs), (ctypes.c_int * n)(*rows),
+                                    M, K, w_bits, stream)
 
 
 def strerror(code: int) -> str:

@@ -22,7 +22,7 @@ import torch
 
 from any_precision_amd import _capi
 
-__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "GEMM_MAX_M"]
+__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "matmul_kbit_group", "GEMM_MAX_M"]
 
 GEMM_MAX_M = _capi.GEMM_MAX_M
 
@@ -84,6 +84,36 @@ def matmul_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_b
                                  w_bits, torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "matmul_kbit")
     return out
+
+
+def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int):
+    """``[matmul_kbit(in_, q, t, w_bits) for q, t in zip(qweights, luts)]`` in one launch: up to
+    GROUP_MAX linears that share the input and the bit-width (q/k/v, gate/up).  No counterpart in
+    the reference; results equal the separate calls bit for bit."""
+    if len(qweights) != len(luts) or not 1 <= len(qweights) <= _capi.GROUP_MAX:
+        raise ValueError(f"matmul_kbit_group: need 1..{_capi.GROUP_MAX} (qweight, lut) pairs")
+    shapes = [_check_weight(q, t, w_bits, "matmul_kbit_group") for q, t in zip(qweights, luts)]
+    K = shapes[0][1]
+    if any(k != K for _, k in shapes):
+        raise ValueError("matmul_kbit_group: all members must have the same in_features")
+    if in_.dtype != torch.float16:
+        raise ValueError(f"matmul_kbit_group: input must be float16, got {in_.dtype}")
+    if any(q.device != in_.device for q in qweights):
+        raise ValueError("matmul_kbit_group: input and weights must be on one device")
+    if in_.dim() < 1 or in_.shape[-1] != K:
+        raise ValueError(f"matmul_kbit_group: input last dim must be K={K}, got {tuple(in_.shape)}")
+    M = in_.numel() // K
+    if M < 1 or M > 8:
+        raise ValueError(f"matmul_kbit_group: batch M={M} outside 1..8")
+    if not in_.is_contiguous():
+        raise ValueError("matmul_kbit_group: input must be contiguous")
+    with torch.cuda.device(in_.device):
+        outs = [torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device) for N, _ in shapes]
+        rc = _capi.matmul_group(in_.data_ptr(), [q.data_ptr() for q in qweights], [t.data_ptr() for t in luts],
+                                [o.data_ptr() for o in outs], [N for N, _ in shapes], M, K, w_bits,
+                                torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "matmul_kbit_group")
+    return outs
 
 
 def gemm_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:

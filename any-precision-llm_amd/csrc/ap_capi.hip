@@ -48,9 +48,14 @@ int check_common(int N, int K, int w_bits) {
     return AP_OK;
 }
 
-int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
-    const int rc = check_common(N, K, w_bits);
-    if (rc != AP_OK) return rc;
+// Launch geometry for `count` linears of n[0..count) rows that share K, M and w_bits.
+int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometry *geo, GemvMembers *mem) {
+    long long rows = 0;
+    for (int g = 0; g < count; g++) {
+        const int rc = check_common(n[g], K, w_bits);
+        if (rc != AP_OK) return rc;
+        rows += n[g];
+    }
     if (M < 1 || M > 8) return AP_EBATCH;
     const Tuning &t = tuning();
     const int W = K >> 5;
@@ -66,12 +71,22 @@ int gemv_geometry(int M, int N, int K, int w_bits, GemvGeometry *geo) {
     // One row per workgroup until that would launch more than target_waves waves, then two
     // (the second row reuses the activation registers; more rows lengthen the compute
     // tail).  From M = 3 on the activations are the larger load: always two rows.
-    int R = t.force_rows > 0 ? t.force_rows : (int)(((long long)N * S + t.target_waves - 1) / t.target_waves);
+    int R = t.force_rows > 0 ? t.force_rows : (int)((rows * S + t.target_waves - 1) / t.target_waves);
     R = (R >= 2 || M > 2) ? 2 : 1;
     geo->wpl = wpl;
     geo->S = S;
     geo->R = R;
-    geo->grid = (N + R - 1) / R;
+    long long grid = 0;
+    for (int g = 0; g < count; g++) {
+        grid += (n[g] + R - 1) / R;
+        if (mem) {
+            mem->n[g] = n[g];
+            mem->wg_end[g] = (int)grid;
+        }
+    }
+    if (grid > 0x7fffffffLL) return AP_ELIMIT;
+    geo->grid = (int)grid;
+    if (mem) mem->count = count;
     return AP_OK;
 }
 
@@ -131,7 +146,7 @@ int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
 
 int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segments, int *rows, int *grid) {
     GemvGeometry geo;
-    const int rc = gemv_geometry(M, N, K, w_bits, &geo);
+    const int rc = gemv_geometry(M, &N, 1, K, w_bits, &geo, nullptr);
     if (rc != AP_OK) return rc;
     if (wpl) *wpl = geo.wpl;
     if (segments) *segments = geo.S;
@@ -186,22 +201,44 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
 
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N,
                    int K, int w_bits, void *stream) {
-    if (!x || !qweight || !lut || !out) return AP_ENULL;
+    return ap_matmul_kbit_group(x, 1, &qweight, &lut, &out, &N, M, K, w_bits, stream);
+}
+
+int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight, const uint16_t *const *lut,
+                         uint16_t *const *out, const int *N, int M, int K, int w_bits, void *stream) {
+    if (!x || !qweight || !lut || !out || !N) return AP_ENULL;
+    if (count < 1 || count > kGemvMaxGroup) return AP_ELIMIT;
+    for (int g = 0; g < count; g++)
+        if (!qweight[g] || !lut[g] || !out[g]) return AP_ENULL;
     GemvGeometry geo;
-    const int rc = gemv_geometry(M, N, K, w_bits, &geo);
+    GemvMembers mem = {};
+    const int rc = gemv_geometry(M, N, count, K, w_bits, &geo, &mem);
     if (rc != AP_OK) return rc;
-    if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
+    if (!aligned16(x)) return AP_EALIGN;
+    for (int g = 0; g < count; g++) {
+        if (!aligned16(qweight[g]) || !aligned16(lut[g])) return AP_EALIGN;
+        mem.qweight[g] = qweight[g];
+        mem.lut[g] = lut[g];
+        mem.out[g] = out[g];
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     // From 5 activation rows on, the MFMA kernel (cost flat in M up to 16 rows) is faster than
-    // the dot-product kernel (cost linear in M) on most shapes and bit-widths.
-    if (M >= tuning().mfma_from_rows) return run_gemm(x, qweight, lut, out, M, N, K, w_bits, st);
+    // the dot-product kernel (cost linear in M) on most shapes and bit-widths; it serves one
+    // linear per launch.
+    if (M >= tuning().mfma_from_rows) {
+        for (int g = 0; g < count; g++) {
+            const int r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
+            if (r != AP_OK) return r;
+        }
+        return AP_OK;
+    }
     switch (w_bits) {
-        case 3: launch_gemv<3>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 4: launch_gemv<4>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 5: launch_gemv<5>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 6: launch_gemv<6>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 7: launch_gemv<7>(M, geo, x, qweight, lut, out, N, K, st); break;
-        default: launch_gemv<8>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 3: launch_gemv<3>(M, geo, x, mem, K, st); break;
+        case 4: launch_gemv<4>(M, geo, x, mem, K, st); break;
+        case 5: launch_gemv<5>(M, geo, x, mem, K, st); break;
+        case 6: launch_gemv<6>(M, geo, x, mem, K, st); break;
+        case 7: launch_gemv<7>(M, geo, x, mem, K, st); break;
+        default: launch_gemv<8>(M, geo, x, mem, K, st); break;
     }
     return launch_status();
 }

@@ -179,18 +179,36 @@ __device__ __forceinline__ void row_dot(const typename WordVec<WPL>::type (&q)[B
 // the planes of its R rows, its activations -- before it computes anything, so the
 // memory pipe is full from the first cycle and there is no loop-carried prefetch.  Every
 // table sits at a compile-time LDS address.
-// Grid: ceil(N / R) workgroups of (64, S) threads; S*64 <= THREADS.  THREADS (256, 512 or
+// Grid: ceil(N / R) workgroups per member, of (64, S) threads; S*64 <= THREADS.  THREADS (256, 512 or
 // 1024) only bounds the workgroup size, so that small workgroups may use more registers
 // per lane (M x WPL x 16 of them hold the activations).
+//
+// One launch serves up to kGemvMaxGroup linears that share x, K and the bit-width (the
+// q/k/v or gate/up projections of a decoder layer): `mem` lists them and the workgroup
+// range of each; a plain call is a set of one.
 template <int BITS, int M, int WPL, int R, int THREADS>
-__global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
-    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight,
-    const half_t *__restrict__ lut, half_t *__restrict__ out, int N, int K) {
+__global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K) {
     constexpr int NC = 1 << BITS;
     constexpr int MAXS = THREADS / kWave;
     typedef typename WordVec<WPL>::type wvec_t;
     __shared__ __attribute__((aligned(16))) uint8_t tables[R][GemvTable<BITS>::kBytes];
     __shared__ float partial[MAXS * R * M];
+
+    // which member this workgroup belongs to (scalar selects; no indexed access to the arguments)
+    const uint32_t *__restrict__ qweight = mem.qweight[0];
+    const half_t *__restrict__ lut = reinterpret_cast<const half_t *>(mem.lut[0]);
+    half_t *__restrict__ out = reinterpret_cast<half_t *>(mem.out[0]);
+    int N = mem.n[0], wg0 = 0;
+#pragma unroll
+    for (int g = 1; g < kGemvMaxGroup; g++) {
+        if (g < mem.count && (int)blockIdx.x >= mem.wg_end[g - 1]) {
+            qweight = mem.qweight[g];
+            lut = reinterpret_cast<const half_t *>(mem.lut[g]);
+            out = reinterpret_cast<half_t *>(mem.out[g]);
+            N = mem.n[g];
+            wg0 = mem.wg_end[g - 1];
+        }
+    }
 
     // blockDim.x is the wave size, so threadIdx.y is wave-uniform: say so, to keep row
     // addresses in scalar registers
@@ -201,7 +219,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(
     const uint32_t w0 = (uint32_t)(s * kWave + lane) * WPL;
     const bool valid = w0 < (uint32_t)W;
     const uint32_t wl = valid ? w0 : 0u;  // lanes past the row end read word 0; their sums are dropped
-    const int row0 = blockIdx.x * R;
+    const int row0 = ((int)blockIdx.x - wg0) * R;
 
     // Issue order matters: the tables first (tiny; staging them to LDS then overlaps the
     // plane loads -- issued last, the table was the last thing to arrive and cost 15-20 %),

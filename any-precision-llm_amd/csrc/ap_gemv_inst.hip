@@ -10,51 +10,46 @@ namespace ap {
 namespace {
 
 template <int BITS, int M, int WPL, int R>
-void launch_rows(const GemvGeometry &geo, const half_t *x, const uint32_t *qweight, const half_t *lut, half_t *out,
-                 int N, int K, hipStream_t stream) {
+void launch_rows(const GemvGeometry &geo, const half_t *x, const GemvMembers &mem, int K, hipStream_t stream) {
     const dim3 block(kWave, geo.S), grid(geo.grid);
     // smallest workgroup bound that holds S waves: leaves the most registers per lane
     if (geo.S <= 4)
-        gemv_kbit_kernel<BITS, M, WPL, R, 256><<<grid, block, 0, stream>>>(x, qweight, lut, out, N, K);
+        gemv_kbit_kernel<BITS, M, WPL, R, 256><<<grid, block, 0, stream>>>(x, mem, K);
     else if (geo.S <= 8)
-        gemv_kbit_kernel<BITS, M, WPL, R, 512><<<grid, block, 0, stream>>>(x, qweight, lut, out, N, K);
+        gemv_kbit_kernel<BITS, M, WPL, R, 512><<<grid, block, 0, stream>>>(x, mem, K);
     else
-        gemv_kbit_kernel<BITS, M, WPL, R, 1024><<<grid, block, 0, stream>>>(x, qweight, lut, out, N, K);
+        gemv_kbit_kernel<BITS, M, WPL, R, 1024><<<grid, block, 0, stream>>>(x, mem, K);
 }
 
 template <int BITS, int M>
-void launch_m(const GemvGeometry &geo, const half_t *x, const uint32_t *qweight, const half_t *lut, half_t *out,
-              int N, int K, hipStream_t stream) {
+void launch_m(const GemvGeometry &geo, const half_t *x, const GemvMembers &mem, int K, hipStream_t stream) {
     if constexpr (M <= 2) {  // two words per lane and one row per workgroup exist for M <= 2 only
         if (geo.wpl == 2) {
-            if (geo.R == 2) return launch_rows<BITS, M, 2, 2>(geo, x, qweight, lut, out, N, K, stream);
-            return launch_rows<BITS, M, 2, 1>(geo, x, qweight, lut, out, N, K, stream);
+            if (geo.R == 2) return launch_rows<BITS, M, 2, 2>(geo, x, mem, K, stream);
+            return launch_rows<BITS, M, 2, 1>(geo, x, mem, K, stream);
         }
-        if (geo.R == 1) return launch_rows<BITS, M, 1, 1>(geo, x, qweight, lut, out, N, K, stream);
+        if (geo.R == 1) return launch_rows<BITS, M, 1, 1>(geo, x, mem, K, stream);
     }
-    launch_rows<BITS, M, 1, 2>(geo, x, qweight, lut, out, N, K, stream);
+    launch_rows<BITS, M, 1, 2>(geo, x, mem, K, stream);
 }
 
 }  // namespace
 
 template <int BITS>
-void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
-                 uint16_t *out, int N, int K, hipStream_t stream) {
-    const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
-    half_t *oh = reinterpret_cast<half_t *>(out);
+void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const GemvMembers &mem, int K, hipStream_t stream) {
+    const half_t *xh = reinterpret_cast<const half_t *>(x);
     switch (M) {
-        case 1: return launch_m<BITS, 1>(geo, xh, qweight, lh, oh, N, K, stream);
-        case 2: return launch_m<BITS, 2>(geo, xh, qweight, lh, oh, N, K, stream);
-        case 3: return launch_m<BITS, 3>(geo, xh, qweight, lh, oh, N, K, stream);
-        case 4: return launch_m<BITS, 4>(geo, xh, qweight, lh, oh, N, K, stream);
-        case 5: return launch_m<BITS, 5>(geo, xh, qweight, lh, oh, N, K, stream);
-        case 6: return launch_m<BITS, 6>(geo, xh, qweight, lh, oh, N, K, stream);
-        case 7: return launch_m<BITS, 7>(geo, xh, qweight, lh, oh, N, K, stream);
-        default: return launch_m<BITS, 8>(geo, xh, qweight, lh, oh, N, K, stream);
+        case 1: return launch_m<BITS, 1>(geo, xh, mem, K, stream);
+        case 2: return launch_m<BITS, 2>(geo, xh, mem, K, stream);
+        case 3: return launch_m<BITS, 3>(geo, xh, mem, K, stream);
+        case 4: return launch_m<BITS, 4>(geo, xh, mem, K, stream);
+        case 5: return launch_m<BITS, 5>(geo, xh, mem, K, stream);
+        case 6: return launch_m<BITS, 6>(geo, xh, mem, K, stream);
+        case 7: return launch_m<BITS, 7>(geo, xh, mem, K, stream);
+        default: return launch_m<BITS, 8>(geo, xh, mem, K, stream);
     }
 }
 
-template void launch_gemv<AP_BITS>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *,
-                                   uint16_t *, int, int, hipStream_t);
+template void launch_gemv<AP_BITS>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
 
 }  // namespace ap

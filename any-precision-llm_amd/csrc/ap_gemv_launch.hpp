@@ -7,25 +7,37 @@
 
 namespace ap {
 
-constexpr int kGemvMaxSeg = 16;  // K-segments (waves) per workgroup
+constexpr int kGemvMaxSeg = 16;    // K-segments (waves) per workgroup
+constexpr int kGemvMaxGroup = 4;   // linears one launch can serve (same x, K, M, w_bits)
+
+// The linears of one launch.  Member g owns workgroups [wg_end[g-1], wg_end[g]); passed to the
+// kernel by value (kernel arguments), so a launch needs no device-side descriptor.
+struct GemvMembers {
+    const uint32_t *qweight[kGemvMaxGroup];
+    const uint16_t *lut[kGemvMaxGroup];
+    uint16_t *out[kGemvMaxGroup];
+    int n[kGemvMaxGroup];       // rows
+    int wg_end[kGemvMaxGroup];  // first workgroup past the member
+    int count;
+};
 
 struct GemvGeometry {
     int wpl;   // words per lane per plane (1 or 2)
     int S;     // K-segments = waves per workgroup
     int R;     // rows per workgroup (1 or 2)
-    int grid;  // workgroups
+    int grid;  // workgroups (of all members together)
 };
 
 // Launches gemv_kbit_kernel<BITS, M, geo.wpl, geo.R, *> on `stream`.  1 <= M <= 8.
 template <int BITS>
-void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const uint32_t *qweight,
-                 const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream);
+void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const GemvMembers &members, int K,
+                 hipStream_t stream);
 
-extern template void launch_gemv<3>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
-extern template void launch_gemv<4>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
-extern template void launch_gemv<5>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
-extern template void launch_gemv<6>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
-extern template void launch_gemv<7>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
-extern template void launch_gemv<8>(int, const GemvGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *, int, int, hipStream_t);
+extern template void launch_gemv<3>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv<4>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv<5>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv<6>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv<7>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv<8>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
 
 }  // namespace ap

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 1
+#define AP_ABI_VERSION 2
 
 enum {
     AP_OK = 0,
@@ -52,6 +52,17 @@ int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
  * reference (main.cu:108).  fp32 accumulation, fp16 result. */
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                    uint16_t *out, int M, int N, int K, int w_bits, void *stream);
+
+/* The GEMVs of `count` (1..4) linears that share x, M, K and w_bits in ONE launch:
+ * out[g][M, N[g]] = x[M,K] . dequant(qweight[g], lut[g])^T.  The arrays are host arrays of
+ * `count` device pointers / row counts.  For the q/k/v and gate/up projections of a decoder
+ * layer, whose launches are otherwise bound by the fixed cost of a kernel launch.  No
+ * counterpart in the reference (its hook for it, fuse_layers, is a stub:
+ * AnyPrecisionForCausalLM.py:168-172); results equal `count` calls of ap_matmul_kbit bit
+ * for bit.  1 <= M <= 8. */
+int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight,
+                         const uint16_t *const *lut, uint16_t *const *out, const int *N,
+                         int M, int K, int w_bits, void *stream);
 
 /* Fused dequant -> MFMA GEMM, 1 <= M <= 128: out[M,N] = x[M,K] . dequant(qweight, lut)^T
  * without materialising the fp16 weight.  No single counterpart in the reference: it is the

@@ -147,3 +147,35 @@ def test_graph_replay_matches_eager(ext):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), rep
+
+
+@pytest.mark.parametrize("K,Ns", [(4096, (512, 128, 128)), (1056, (33, 7, 64, 5)), (11008, (96, 96)), (96, (3,))])
+def test_group_launch_equals_separate_calls_bit_for_bit(ext, oracle, K, Ns):
+    layers = [make(N, K, seed=40 + i) for i, N in enumerate(Ns)]
+    gpu = [layer_to_gpu(L) for L in layers]
+    for b in (3, 4, 5, 8):
+        for M in (1, 2, 3, 4, 6):      # 6: the members go through the MFMA kernel one by one
+            print(f"group K={K} Ns={Ns} b={b} M={M}", flush=True)
+            x, xg = _x(M, K, seed=M)
+            outs = ext.matmul_kbit_group(xg, [q for q, _ in gpu], [luts[b] for _, luts in gpu], b)
+            assert len(outs) == len(Ns)
+            for (q, luts), L, got in zip(gpu, layers, outs):
+                assert got.shape == (M, L.N)
+                single = ext.matmul_kbit(xg, q, luts[b], b)
+                assert torch.equal(got, single)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                assert_close_gemv(got, want, f"K={K} N={L.N} b={b} M={M}")
+
+
+def test_group_argument_errors(ext):
+    L = make(8, 64, seed=0)
+    q, luts = layer_to_gpu(L)
+    _, xg = _x(1, 64)
+    with pytest.raises(ValueError):
+        ext.matmul_kbit_group(xg, [q] * 5, [luts[3]] * 5, 3)          # more members than a launch holds
+    with pytest.raises(ValueError):
+        ext.matmul_kbit_group(xg, [q, q], [luts[3]], 3)
+    L2 = make(8, 96, seed=1)
+    q2, luts2 = layer_to_gpu(L2)
+    with pytest.raises(ValueError):
+        ext.matmul_kbit_group(xg, [q, q2], [luts[3], luts2[3]], 3)    # different in_features
