@@ -7,7 +7,8 @@ not by the kernels.  Here one decode step -- embedding, 32 x (norm, q/k/v GEMV, 
 cache write, attention over a static cache, o GEMV, norm, gate/up GEMV, SiLU, down GEMV),
 final norm, head, argmax, position increment -- is recorded once per precision and replayed
 per token: no host work between tokens.  Only the seven linears per layer are this
-library's kernels; everything else is stock PyTorch ops, as in the reference.
+library's kernels (q/k/v and gate/up as one grouped launch each); everything else is stock
+PyTorch ops, as in the reference.
 
 Supports Llama-style decoders (RMSNorm, rotary attention with optional grouped KV heads,
 SwiGLU MLP, no biases in norms); anything else raises.
@@ -19,6 +20,8 @@ import math
 import torch
 import torch.nn.functional as F
 
+from .linear import forward_group
+
 
 def _rotate_half(x):
     h = x.shape[-1] // 2
@@ -26,7 +29,9 @@ def _rotate_half(x):
 
 
 class GraphDecoder:
-    def __init__(self, ap_model, max_len=512):
+    def __init__(self, ap_model, max_len=512, group_launches=True):
+        """``group_launches``: issue the q/k/v and the gate/up GEMVs of a layer as one launch each."""
+        self.group_launches = group_launches
         cfg = ap_model.config
         if getattr(cfg, "model_type", None) != "llama":
             raise NotImplementedError(f"GraphDecoder handles Llama-architecture models, got {cfg.model_type!r}")
@@ -67,6 +72,11 @@ class GraphDecoder:
         self.stream = torch.cuda.Stream(device=dev)
 
     # ------------------------------------------------------------------ the network
+    def _group(self, modules, x, precision):
+        if self.group_launches:
+            return forward_group(modules, x, precision)
+        return [m(x, precision=precision) for m in modules]
+
     def _norm(self, x, w):
         return F.rms_norm(x, (x.shape[-1],), w, self.eps)
 
@@ -75,9 +85,9 @@ class GraphDecoder:
         layer = self.layers[li]
         T = h.shape[0]
         x = self._norm(h, layer.input_layernorm.weight)
-        q = layer.self_attn.q_proj(x, precision=precision).view(T, self.nh, self.hd)
-        k = layer.self_attn.k_proj(x, precision=precision).view(T, self.nkv, self.hd)
-        v = layer.self_attn.v_proj(x, precision=precision).view(T, self.nkv, self.hd)
+        att_in = layer.self_attn
+        q, k, v = self._group((att_in.q_proj, att_in.k_proj, att_in.v_proj), x, precision)
+        q, k, v = q.view(T, self.nh, self.hd), k.view(T, self.nkv, self.hd), v.view(T, self.nkv, self.hd)
         q = q * cos + _rotate_half(q) * sin
         k = k * cos + _rotate_half(k) * sin
         self.kcache[li].index_copy_(1, pos_idx, k.transpose(0, 1))
@@ -90,8 +100,7 @@ class GraphDecoder:
         att = torch.bmm(probs, self.vcache[li]).view(self.nh, T, self.hd).transpose(0, 1).reshape(T, self.nh * self.hd)
         h = h + layer.self_attn.o_proj(att, precision=precision)
         x = self._norm(h, layer.post_attention_layernorm.weight)
-        gate = layer.mlp.gate_proj(x, precision=precision)
-        up = layer.mlp.up_proj(x, precision=precision)
+        gate, up = self._group((layer.mlp.gate_proj, layer.mlp.up_proj), x, precision)
         return h + layer.mlp.down_proj(F.silu(gate) * up, precision=precision)
 
     def _forward(self, tokens, pos_idx, precision):
@@ -122,9 +131,10 @@ class GraphDecoder:
         T = ids.numel()
         if T < 1 or T >= self.max_len:
             raise ValueError(f"prompt length {T} outside 1..{self.max_len - 1}")
-        self.kcache.zero_()
-        self.vcache.zero_()
+        self.stream.wait_stream(torch.cuda.current_stream(self.dev))     # the ids may still be in flight there
         with torch.cuda.stream(self.stream):
+            self.kcache.zero_()
+            self.vcache.zero_()
             pos_idx = torch.arange(T, device=self.dev)
             logits = self._forward(ids, pos_idx, precision)
             self.logits.copy_(logits)

@@ -14,15 +14,32 @@ import torch
 import torch.nn as nn
 
 try:
-    from any_precision_ext import matmul_kbit, dequant_kbit, gemm_kbit, GEMM_MAX_M
+    from any_precision_ext import matmul_kbit, matmul_kbit_group, dequant_kbit, gemm_kbit, GEMM_MAX_M
 except ModuleNotFoundError:
-    matmul_kbit, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, 0
+    matmul_kbit, matmul_kbit_group, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, None, 0
 
 
 # Up to this many activation rows the fused GEMM beats dequant_kbit + torch.matmul on every
 # Llama-2-7B shape and bit-width measured (1.3-2.6x at 16 rows); beyond, the re-read of the
 # activations per 16 weight rows costs more than materialising the weight once.
 FUSED_GEMM_ROWS = min(32, GEMM_MAX_M)
+
+
+def forward_group(modules, x, precision=None):
+    """``[m(x, precision=precision) for m in modules]`` for linears that share their input (the
+    q/k/v or gate/up projections of a decoder layer).  Up to 4 activation rows and 4 modules
+    the GEMVs go out as ONE launch; otherwise module by module.  The reference has no
+    counterpart (its ``fuse_layers`` is a stub, AnyPrecisionForCausalLM.py:168-172)."""
+    rows = x.numel() // x.shape[-1]
+    w_bits = modules[0].precision if precision is None else precision
+    if rows > 4 or not 2 <= len(modules) <= 4 or not x.is_contiguous() or any(
+            m.in_features != modules[0].in_features for m in modules):
+        return [m(x, precision=w_bits) for m in modules]
+    outs = matmul_kbit_group(x, [m.qweight for m in modules], [m._buffers[f"lut{w_bits}"] for m in modules], w_bits)
+    for m, o in zip(modules, outs):
+        if m.bias is not None:
+            o += m.bias
+    return outs
 
 
 class AnyPrecisionLinear(nn.Module):

@@ -34,12 +34,14 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--workload", default="llama2_7b_layer_batch1",
                     choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model",
-                             "llama2_7b_decode"),
+                             "llama2_7b_decode", "llama2_7b_prefill"),
                     help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
                          "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
                          "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.  "
                          "llama2_7b_decode: batch-1 greedy decoding of a random-init Llama-2-7B-shaped model, "
-                         "256 tokens after a 128-token prompt, per w_bits.")
+                         "256 tokens after a 128-token prompt, per w_bits.  "
+                         "llama2_7b_prefill: the seven linears of a layer on 32 x 512 = 16384 activation rows "
+                         "(dequant_kbit + library GEMM, the large-batch branch of AnyPrecisionLinear).")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -91,6 +93,8 @@ def main():
         return batch_sweep(args, torch, _capi, synth)
     if args.workload == "llama2_7b_dequant_full_model":
         return dequant_full_model(args, torch, _capi, synth)
+    if args.workload == "llama2_7b_prefill":
+        return prefill_linears(args, torch, _capi, synth)
     if args.workload == "llama2_7b_decode":
         with torch.inference_mode():     # the decoder captures its graphs in inference mode; stay in it
             return decode_tokens(args, torch, _capi, synth)
@@ -128,9 +132,9 @@ def main():
         if rc != 0:
             raise RuntimeError(_capi.strerror(rc))
 
-    def time_graph(enqueue, reps):
-        """us per call of `enqueue(stream)`: `reps` calls captured in one HIP graph, second replay timed
-        (with --eager: launched one by one, host launch cost included)."""
+    def time_graph(enqueue, reps, replays=5):
+        """us per call of `enqueue(stream)`: `reps` calls captured in one HIP graph; median over `replays`
+        timed replays after an untimed one (with --eager: launched one by one, host launch cost included)."""
         with torch.cuda.stream(side):
             if args.eager:
                 enqueue(side.cuda_stream)
@@ -148,12 +152,17 @@ def main():
                     enqueue(torch.cuda.current_stream().cuda_stream)
             g.replay()
             side.synchronize()
-            a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a0.record(side)
-            g.replay()
-            a1.record(side)
-            side.synchronize()
-        return a0.elapsed_time(a1) * 1e3 / reps
+            times = []
+            for _ in range(replays):
+                a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a0.record(side)
+                g.replay()
+                a1.record(side)
+                side.synchronize()
+                times.append(a0.elapsed_time(a1) * 1e3 / reps)
+        times.sort()
+        time_graph.spread = (times[0], times[-1])
+        return times[len(times) // 2]
 
     def step(i: int, stream: int):
         for b in BITS:
@@ -161,6 +170,29 @@ def main():
                 launch(N, K, b, stream)
 
     step_bytes = sum(synth.gemv_bytes(N, K, b, 1) for _, N, K in shapes for b in BITS)
+
+    # the same 42 GEMVs with the linears that share an input issued as one launch each (q,k,v; gate,up):
+    # 24 launches per step.  Reported beside the headline, which stays one launch per linear.
+    names = [n for n, _, _ in shapes]
+    groups = [[names.index(n) for n in g] for g in (("q_proj", "k_proj", "v_proj"), ("o_proj",),
+                                                    ("gate_proj", "up_proj"), ("down_proj",))]
+    lin_out = [torch.empty((1, N), dtype=torch.float16, device="cuda") for _, N, _ in shapes]
+
+    def grouped_step(stream: int):
+        for b in BITS:
+            for g in groups:
+                qs, ts = [], []
+                for li in g:
+                    _, N, K = shapes[li]
+                    P = pools[(N, K)]
+                    j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
+                    qs.append(P.qweight[j].data_ptr())
+                    ts.append(P.luts[b][j].data_ptr())
+                K = shapes[g[0]][2]
+                rc = _capi.matmul_group(xb[(1, K)].data_ptr(), qs, ts, [lin_out[li].data_ptr() for li in g],
+                                        [shapes[li][1] for li in g], 1, K, b, stream)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
 
     if args.calibrate_copy:
         src = torch.ones(64 << 20, dtype=torch.int32, device="cuda")      # 256 MiB
@@ -198,15 +230,26 @@ def main():
     ms_per_step = total_ms / args.steps
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
+    grouped = None
+    if not args.eager and not args.only_step:
+        us = time_graph(grouped_step, max(2, args.steps // 2))
+        grouped = {"launches_per_step": len(BITS) * len(groups), "ms_per_step": round(us / 1e3, 5),
+                   "GBps": round(step_bytes / us / 1e3, 1), "frac": round(step_bytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                   "note": "same 42 GEMVs, q/k/v and gate/up each as one ap_matmul_kbit_group launch"}
+
     # ---- per-kernel table: each (shape, w_bits) alone, rotating over the pool (cold planes)
     table, dequant_table, batch_table = [], [], []
     if not args.only_step:
         for (N, K), idxs in uniq.items():
             for b in BITS:
-                us = time_graph(lambda st: launch(N, K, b, st), args.kernel_reps)
                 by = synth.gemv_bytes(N, K, b, 1)
+                # enough launches that a replay streams >= 1 GB before it returns to its first weight set
+                reps = min(pools[(N, K)].sets, max(args.kernel_reps, int(1e9 / by) + 1))
+                us = time_graph(lambda st: launch(N, K, b, st), reps)
                 geo = _capi.matmul_geometry(1, N, K, b)
-                table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 3), "GBps": round(by / us / 1e3, 1),
+                lo, hi = getattr(time_graph, "spread", (us, us))
+                table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 3), "us_min": round(lo, 3),
+                              "us_max": round(hi, 3), "GBps": round(by / us / 1e3, 1),
                               "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": by,
                               "count_in_step": len(idxs), "geometry": geo})
 
@@ -279,6 +322,36 @@ def main():
         cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
                "sample": "C oracle GEMV (unpack+gather+fp32 dot, OpenMP over rows): 4096x4096, 11008x4096, "
                          "4096x11008 at w_bits 3 and 8, batch 1, mean of 3 runs each"}
+        # the same semantics written with PyTorch CPU ops (bitplane unpack -> table gather -> matmul), 4096x4096
+        N = K = 4096
+        nthr = torch.get_num_threads()
+        qw_t = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(8, N, K // 32), dtype=np.int64).astype(np.int32))
+        x_t = torch.from_numpy(rng.normal(0, 1, size=(1, K)).astype(np.float32))
+
+        def torch_unpack(b):
+            by = qw_t[:b].contiguous().view(torch.uint8).view(b, N, K // 1024, 32, 4).flip(-1)        # [p,n,c,t,j]
+            bits = (by.unsqueeze(-1) >> torch.arange(7, -1, -1, dtype=torch.uint8)) & 1                  # [p,n,c,t,j,e]
+            bits = bits.permute(0, 1, 2, 4, 3, 5).reshape(b, N, K)
+            w = (1 << torch.arange(b - 1, -1, -1, dtype=torch.int64)).view(b, 1, 1)
+            return (bits.to(torch.int64) * w).sum(0)
+
+        t_e2e, t_mm, by_t = 0.0, 0.0, 0
+        for b in cpu_bits:
+            lut_t = torch.from_numpy(np.sort(rng.normal(0, 0.02, size=(N, 1 << b)), axis=1).astype(np.float32))
+            t0 = time.perf_counter()
+            wdq = torch.gather(lut_t, 1, torch_unpack(b))
+            y = x_t @ wdq.T
+            t_e2e += time.perf_counter() - t0
+            t0 = time.perf_counter()
+            for _ in range(5):
+                y = x_t @ wdq.T
+            t_mm += (time.perf_counter() - t0) / 5
+            by_t += synth.gemv_bytes(N, K, b, 1)
+        cpu["torch_reference_semantics"] = {
+            "GBps_end_to_end": round(by_t / t_e2e / 1e9, 4), "ms_end_to_end": round(t_e2e * 1e3 / len(cpu_bits), 1),
+            "ms_matmul_only": round(t_mm * 1e3 / len(cpu_bits), 3), "threads": nthr,
+            "sample": "torch CPU ops, 4096x4096, w_bits 3 and 8, batch 1: unpack + gather + matmul once; matmul "
+                      "alone on the dequantised fp32 weight, mean of 5"}
 
     result = {
         "metric": "bitplane GEMV effective HBM GB/s, Llama-2-7B layer set, w_bits 3-8, batch 1",
@@ -290,7 +363,7 @@ def main():
                    "weight_sets_per_shape": {f"{N}x{K}": P.sets for (N, K), P in pools.items()},
                    "bytes_per_step": step_bytes,
                    "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "layers": table,
+        "roofline": roofline, "cpu_baseline": cpu, "grouped_launches": grouped, "layers": table,
         "dequant_kbit": dequant_table, "batch_us": batch_table,
     }
     if args.table and table:
@@ -438,6 +511,7 @@ def decode_tokens(args, torch, _capi, synth):
     model = AnyPrecisionForCausalLM.from_config(cfg, seed=0, device="cuda")
     prompt_len, new_tokens = 128, 256
     dec = GraphDecoder(model, max_len=prompt_len + new_tokens + 8)
+    dec_single = GraphDecoder(model, max_len=prompt_len + new_tokens + 8, group_launches=False)
     ids = torch.randint(0, cfg.vocab_size, (prompt_len,), generator=torch.Generator().manual_seed(0)).cuda()
     lib = _capi.lib
     side = torch.cuda.Stream()
@@ -452,6 +526,16 @@ def decode_tokens(args, torch, _capi, synth):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         tok_s = (new_tokens - 9) / dt
+        single = None
+        if b in (3, 8):
+            dec_single.prefill(ids, b)
+            dec_single.capture(b)
+            dec_single.decode(8, b)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dec_single.decode(64, b)
+            torch.cuda.synchronize()
+            single = 64 / (time.perf_counter() - t0)
         eager = None
         if b in (3, 8):
             dec.prefill(ids, b)
@@ -475,6 +559,7 @@ def decode_tokens(args, torch, _capi, synth):
         lin_bytes = sum(synth.gemv_bytes(l.out_features, l.in_features, b, 1) for l in model.ap_linears)
         rows.append({"w_bits": b, "tokens_per_s": round(tok_s, 1), "ms_per_token": round(1e3 / tok_s, 3),
                      "eager_tokens_per_s": None if eager is None else round(eager, 1),
+                     "one_launch_per_linear_tokens_per_s": None if single is None else round(single, 1),
                      "linears_ms_per_token": round(lin_us / 1e3, 3),
                      "linears_GBps": round(lin_bytes / lin_us / 1e3, 1),
                      "linears_frac_of_hbm_peak": round(lin_bytes / lin_us / 1e3 / HBM_PEAK_GBS, 4)})
@@ -486,6 +571,55 @@ def decode_tokens(args, torch, _capi, synth):
         "config": {"workload": f"greedy decode of {new_tokens} tokens after a {prompt_len}-token prompt, batch 1, "
                                "32 layers / hidden 4096 / FFN 11008 / 32 heads / vocab 32000; decode step replayed "
                                "from one HIP graph; linears = this library, everything else stock PyTorch ops"},
+        "per_w_bits": rows}))
+
+
+
+def prefill_linears(args, torch, _capi, synth):
+    """The seven linears of a Llama-2-7B layer on M = 32 x 512 activation rows through AnyPrecisionLinear's
+    large-batch branch: dequant_kbit to fp16, then the library GEMM.  Reports the share of the dequant."""
+    from any_precision_amd import AnyPrecisionLinear
+    import any_precision_ext as ext
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    M = 32 * 512
+    side = torch.cuda.Stream()
+    rows = []
+    with torch.inference_mode():
+        for b in (3, 8):
+            t_total = t_deq = flops = 0.0
+            for name, N, K in synth.LLAMA2_7B_LAYER:
+                lin = AnyPrecisionLinear(K, N, list(range(3, 9)), bias=False, device="cuda", dtype=torch.float16)
+                lin.qweight.copy_(torch.randint(-2**31, 2**31 - 1, lin.qweight.shape, dtype=torch.int32, device="cuda",
+                                                generator=gen))
+                lin._buffers[f"lut{b}"].copy_(torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02,
+                                                         dim=1).values.half())
+                x = torch.randn((M, K), device="cuda", generator=gen).half()
+
+                def run(fn, reps=5):
+                    with torch.cuda.stream(side):
+                        fn()
+                        side.synchronize()
+                        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        a0.record(side)
+                        for _ in range(reps):
+                            fn()
+                        a1.record(side)
+                        side.synchronize()
+                    return a0.elapsed_time(a1) / reps
+                t_total += run(lambda: lin(x, precision=b))
+                t_deq += run(lambda: ext.dequant_kbit(lin.qweight, lin._buffers[f"lut{b}"], b))
+                flops += 2.0 * M * N * K
+                del lin, x
+            rows.append({"w_bits": b, "ms_per_layer_linears": round(t_total, 3), "ms_dequant": round(t_deq, 3),
+                         "dequant_share": round(t_deq / t_total, 4), "TFLOPs": round(flops / t_total / 1e9, 1)})
+    print(json.dumps({
+        "metric": "prefill linears TFLOP/s, Llama-2-7B layer set, 16384 activation rows",
+        "value": round(sum(r["TFLOPs"] for r in rows) / len(rows), 1), "unit": "TFLOP/s", "n_gpus": 1,
+        "higher_is_better": True, "vs_baseline": None, "dtype": "fp16 (library GEMM) on dequantised weights",
+        "data": "synthetic",
+        "config": {"workload": "7 linears of a Llama-2-7B decoder layer, M = 32 x 512 rows, dequant_kbit + "
+                               "torch.matmul per call (weight rebuilt on every call), eager launches"},
         "per_w_bits": rows}))
 
 

@@ -75,6 +75,8 @@ def test_graph_decoder_matches_eager_and_the_dense_model(pair):
         again = dec.generate(ids, 12, precision=b, use_graph=True)     # replays after eager work in between
         assert with_graph.shape == (21,) and torch.equal(with_graph[:9], ids)
         assert torch.equal(with_graph, eager) and torch.equal(with_graph, again)
+        ungrouped = GraphDecoder(ap, max_len=64, group_launches=False).generate(ids, 12, precision=b)
+        assert torch.equal(with_graph, ungrouped)       # grouped launches give the same bits
         # the logits that chose the last token, against the dense model on the same prefix
         with torch.inference_mode():
             want = dense[b](with_graph[:-1].unsqueeze(0)).logits[0, -1]
