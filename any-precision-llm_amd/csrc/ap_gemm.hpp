@@ -56,7 +56,7 @@ __device__ __forceinline__ void transpose_rows4(uint32_t (&r)[4]) {
 }
 
 // MB = activation row blocks of 16 (M <= 16*MB).  Grid: ceil(N/16) workgroups of (64, KS).
-template <int BITS, int MB, bool VEC4>
+template <int BITS, int MB, bool VEC4, int MP>
 __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K) {
@@ -65,6 +65,9 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     constexpr int TQ = kGemmRows * NC / 8;  // 16-byte quads of the 16 tables
     __shared__ __attribute__((aligned(16))) half_t tables[kGemmRows][NC];
     __shared__ float red[kGemmMaxSplit][MB][4][kWave];
+    // activation staging, one private region per wave: MP rows x 16 octets (4 byte groups x 4 words)
+    __shared__ u32x4 xs[kGemmMaxSplit][MP > 0 ? MP * 16 : 1];
+    static_assert(MP == 0 || (MP >= 8 && MP <= 16 * MB && (MP & (MP - 1)) == 0), "");
 
     const int lane = threadIdx.x;
     const int ks = __builtin_amdgcn_readfirstlane(threadIdx.y), KS = blockDim.y;
@@ -132,10 +135,18 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     // step may reach past the end of the row (only the last step of a row can).
     //
     // The unit of the inner schedule is the octet (one byte group of one word: one B operand,
-    // MB MFMAs).  The activations of an octet come from L2 and nothing else in the wave can
-    // hide that latency, so they are requested AHEAD octets before they are used.
+    // MB MFMAs).  Its A operand is 16 bytes of x per lane, lane (m, g) taking row m and the
+    // g-th octet of a 64-byte run.  Every workgroup reads its K-slices of ALL of x, so the
+    // activations are re-read N/16 times from L2 -- (N/16) * M * K * 2 bytes, more than the
+    // planes from M = 2 * w_bits rows on -- and that traffic, not HBM, bounds the kernel.
+    // MP == 0: the operands are loaded straight from global memory, AHEAD octets early.
+    // MP > 0: the wave loads the x block of a word group (MP rows x 4 runs of 64 bytes) with
+    // adjacent lanes on adjacent addresses, parks it in its own LDS region and reads the
+    // operands from there (slots skewed by the octet index so that writes and reads are free
+    // of bank conflicts; LDS operations of one wave complete in order, so no barrier).
     constexpr int OCT = 4 * WPS;
     constexpr int AHEAD = MB == 1 ? 4 : (MB == 2 ? 2 : 1);
+    constexpr int NL = MP / 4;  // staging loads per lane and word group
     auto process = [&](auto check_c, int step, uint32_t(&q)[BITS][WPS]) {
         constexpr bool CHECK = decltype(check_c)::value;
         // x byte offset of byte group 0 of each word, and the distance between byte groups
@@ -150,16 +161,45 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
             kb[wi] = ((uint32_t)chunk << 11) + ((uint32_t)(wc & 31) << 4);
             jstride[wi] = chunk == full_chunks ? tail_stride : 512u;
         }
-        half8_t a[OCT][MB];
+
+        // ---- direct path (MP == 0): fragments from global memory, AHEAD octets early
+        half8_t a[MP == 0 ? OCT : 1][MB];
         auto load_a = [&](auto t_c) {
             constexpr int t = decltype(t_c)::value;
-            if constexpr (t < OCT) {
+            if constexpr (MP == 0 && t < OCT) {
                 const uint32_t koff = kb[t / 4] + (uint32_t)(t % 4) * jstride[t / 4];
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
                     a[t][mb] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(x) + (size_t)(xoff[mb] + koff));
             }
         };
+        // ---- staged path (MP > 0): lane = (row r + 4 i, byte group sj, octet sg of the run)
+        const int sg = lane & 3, sj = (lane >> 2) & 3, sr = lane >> 4;
+        u32x4 xr[NL > 0 ? NL : 1];
+        auto stage_load = [&](int wi) {
+            if constexpr (MP > 0) {
+                int w = 4 * (WPS * step + wi) + sg;
+                if (CHECK) w = min(w, W - 1);
+                const int chunk = w >> 5;
+                const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)(w & 31) << 4) +
+                                      (uint32_t)sj * (chunk == full_chunks ? tail_stride : 512u);
+#pragma unroll
+                for (int i = 0; i < NL; i++) {
+                    const uint32_t roff = (uint32_t)min(sr + 4 * i, M - 1) * (uint32_t)K * 2u;
+                    xr[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + (size_t)(roff + koff));
+                }
+            }
+        };
+        auto stage_store = [&]() {
+            if constexpr (MP > 0) {
+                const int o = 4 * sj + sg;
+#pragma unroll
+                for (int i = 0; i < NL; i++) xs[ks][o * MP + ((sr + 4 * i + o) & (MP - 1))] = xr[i];
+                __builtin_amdgcn_wave_barrier();
+            }
+        };
+
+        if constexpr (MP > 0) stage_load(0);
         static_for<AHEAD>([&](auto t_c) { load_a(t_c); });
         if constexpr (VEC4) {
 #pragma unroll
@@ -172,6 +212,10 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
             constexpr int t = decltype(t_c)::value, wi = t / 4, j = t % 4, c = 3 - j;
             load_a(std::integral_constant<int, t + AHEAD>{});
             if constexpr (j == 0) {
+                if constexpr (MP > 0) {
+                    stage_store();
+                    if constexpr (wi + 1 < WPS) stage_load(wi + 1);
+                }
                 uint32_t qq[BITS];
 #pragma unroll
                 for (int p = 0; p < BITS; p++) qq[p] = q[p][wi];
@@ -197,8 +241,17 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
             });
             const half8_t bfrag = __builtin_bit_cast(half8_t, bw);
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[t][mb], bfrag, acc[mb], 0, 0, 0);
+            for (int mb = 0; mb < MB; mb++) {
+                half8_t afrag;
+                if constexpr (MP > 0) {
+                    const int o = 4 * j + grp;
+                    const int m = (mb * 16 + col) & (MP - 1);  // MP < 16: rows repeat, their results are not stored
+                    afrag = __builtin_bit_cast(half8_t, xs[ks][o * MP + ((m + o) & (MP - 1))]);
+                } else {
+                    afrag = a[t][mb];
+                }
+                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag, acc[mb], 0, 0, 0);
+            }
         });
     };
 

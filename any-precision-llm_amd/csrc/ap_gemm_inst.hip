@@ -15,16 +15,24 @@ void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qwe
     half_t *oh = reinterpret_cast<half_t *>(out);
     const dim3 block(kWave, geo.ks), grid(geo.grid);
     const bool vec4 = ((K >> 5) & 3) == 0;  // whole 16-byte quads of words per row
-#define AP_GEMM_CASE(MBV)                                                                                   \
-    case MBV:                                                                                               \
-        if (vec4) gemm_kbit_kernel<BITS, MBV, true><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);  \
-        else gemm_kbit_kernel<BITS, MBV, false><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);      \
-        break;
+    // Two row blocks (17..32 activation rows) stage the activations through LDS (measured
+    // 10-17 % faster at every bit-width); one row block is as fast or faster straight from
+    // global memory, and beyond two the staging region would crowd out the second workgroup
+    // of a CU.
+#define AP_GEMM_LAUNCH(MBV, MPV)                                                                                  \
+    do {                                                                                                          \
+        if (vec4) gemm_kbit_kernel<BITS, MBV, true, MPV><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);   \
+        else gemm_kbit_kernel<BITS, MBV, false, MPV><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);       \
+    } while (0)
+#define AP_GEMM_CASE(MBV) \
+    case MBV: AP_GEMM_LAUNCH(MBV, 0); break;
     switch (geo.mb) {
-        AP_GEMM_CASE(1) AP_GEMM_CASE(2) AP_GEMM_CASE(3) AP_GEMM_CASE(4)
-        AP_GEMM_CASE(5) AP_GEMM_CASE(6) AP_GEMM_CASE(7)
-        default: AP_GEMM_CASE(8)
+        AP_GEMM_CASE(1)
+        case 2: AP_GEMM_LAUNCH(2, 32); break;
+        AP_GEMM_CASE(3) AP_GEMM_CASE(4) AP_GEMM_CASE(5) AP_GEMM_CASE(6) AP_GEMM_CASE(7)
+        default: AP_GEMM_LAUNCH(8, 0); break;
     }
+#undef AP_GEMM_LAUNCH
 #undef AP_GEMM_CASE
 }
 
