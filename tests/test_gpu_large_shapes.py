@@ -1,0 +1,48 @@
+"""Largest shapes of the Llama family (70B MLP: 28672 x 8192 and 8192 x 28672) against a
+reference written with torch ops on the GPU straight from the layout definition
+(pack.py:51-68: element k of row n sits in word 32 c + t, byte group j, bit e with
+k = 1024 c + 8 (32 j + t) + e) -- independent of the oracle and of the kernels' code, and big
+enough to catch 32-bit overflow in the addressing."""
+import pytest
+import torch
+
+from _util import REL_TOL
+
+pytestmark = pytest.mark.gpu
+
+
+def torch_indices(qweight, b):
+    """int64 [N, K] index of every element from planes 0..b-1 (K a multiple of 1024)."""
+    P, N, W = qweight.shape
+    K = W * 32
+    idx = torch.zeros((N, K), dtype=torch.int64, device=qweight.device)
+    shifts = torch.arange(31, -1, -1, device=qweight.device, dtype=torch.int64)       # bit of (j, e), MSB first
+    for p in range(b):
+        words = qweight[p].to(torch.int64) & 0xFFFFFFFF                              # [N, W]
+        bits = (words.unsqueeze(-1) >> shifts) & 1                                    # [N, W, (j e)]
+        bits = bits.view(N, K // 1024, 32, 4, 8).permute(0, 1, 3, 2, 4).reshape(N, K)  # [n, c, j, t, e]
+        idx |= bits << (b - 1 - p)
+        del words, bits
+    return idx
+
+
+@pytest.mark.parametrize("N,K", [(28672, 8192), (8192, 28672)])
+def test_llama70b_mlp_shapes(N, K):
+    import any_precision_ext as ext
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(N)
+    q = torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda", generator=gen)
+    for b in (3, 8):
+        print(f"large N={N} K={K} b={b}", flush=True)
+        lut = torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02, dim=1).values.half()
+        want_w = torch.gather(lut, 1, torch_indices(q, b))
+        got_w = ext.dequant_kbit(q, lut, b)
+        assert torch.equal(got_w, want_w), f"dequant N={N} K={K} b={b}"
+        del got_w
+        for M, fn in ((1, ext.matmul_kbit), (4, ext.matmul_kbit), (8, ext.matmul_kbit), (32, ext.gemm_kbit)):
+            x = torch.randn((M, K), device="cuda", generator=gen).half()
+            want = x.double() @ want_w.double().T
+            got = fn(x, q, lut, b).double()
+            assert (got - want).norm() <= REL_TOL * want.norm(), f"{fn.__name__} M={M} b={b}"
+            assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"{fn.__name__} M={M} b={b}"
+        del want_w
