@@ -58,6 +58,7 @@ def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 8) -> str:
     for b in range(3, 9):
         units.append((os.path.join(CSRC, "ap_gemv_inst.hip"), os.path.join(OBJDIR, f"ap_gemv_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemm_inst.hip"), os.path.join(OBJDIR, f"ap_gemm_b{b}.o"), [f"-DAP_BITS={b}"]))
+        units.append((os.path.join(CSRC, "ap_gemv4_inst.hip"), os.path.join(OBJDIR, f"ap_gemv4_b{b}.o"), [f"-DAP_BITS={b}"]))
     hipcc = _hipcc()
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(lambda u: _run([hipcc, *compile_flags, *u[2], u[0], "-o", u[1]], verbose), units))

@@ -1,0 +1,48 @@
+// 4x4x4 matrix-core skinny GEMM kernels of one bit-width (compile with -DAP_BITS=3..8) and
+// their launch dispatch.
+#include "ap_gemv4.hpp"
+
+#ifndef AP_BITS
+#error "compile with -DAP_BITS=<3..8>"
+#endif
+
+namespace ap {
+namespace {
+
+template <int BITS, int MG, int G, int RQ>
+void launch_rq(const Gemv4Geometry &geo, const half_t *x, const uint32_t *qweight, const half_t *lut, half_t *out,
+              int M, int N, int K, hipStream_t stream) {
+    const dim3 block(kWave, geo.S), grid(geo.grid);
+    // smallest workgroup bound that holds S waves
+    if (geo.S <= 4)
+        gemv4_kbit_kernel<BITS, MG, G, RQ, 256><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+    else if (geo.S <= 8)
+        gemv4_kbit_kernel<BITS, MG, G, RQ, 512><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+    else
+        gemv4_kbit_kernel<BITS, MG, G, RQ, 1024><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+}
+
+template <int BITS, int MG>
+void launch_mg(const Gemv4Geometry &geo, const half_t *x, const uint32_t *qweight, const half_t *lut, half_t *out,
+               int M, int N, int K, hipStream_t stream) {
+    switch (geo.G) {  // two row quads per workgroup measured best; other counts are not instantiated
+        case 1: return launch_rq<BITS, MG, 1, 2>(geo, x, qweight, lut, out, M, N, K, stream);
+        case 2: return launch_rq<BITS, MG, 2, 2>(geo, x, qweight, lut, out, M, N, K, stream);
+        default: return launch_rq<BITS, MG, 4, 2>(geo, x, qweight, lut, out, M, N, K, stream);
+    }
+}
+
+}  // namespace
+
+template <int BITS>
+void launch_gemv4(const Gemv4Geometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                  uint16_t *out, int M, int N, int K, hipStream_t stream) {
+    const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
+    half_t *oh = reinterpret_cast<half_t *>(out);
+    launch_mg<BITS, 1>(geo, xh, qweight, lh, oh, M, N, K, stream);  // one group of four activation rows
+}
+
+template void launch_gemv4<AP_BITS>(const Gemv4Geometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *,
+                                    int, int, int, hipStream_t);
+
+}  // namespace ap

@@ -179,3 +179,36 @@ def test_group_argument_errors(ext):
     q2, luts2 = layer_to_gpu(L2)
     with pytest.raises(ValueError):
         ext.matmul_kbit_group(xg, [q, q2], [luts[3], luts2[3]], 3)    # different in_features
+
+
+def test_every_kernel_for_small_batches_agrees_with_the_oracle(oracle):
+    """ap_matmul_kbit picks between the dot-product kernel and the 4x4x4 matrix-core kernel by
+    shape and bit-width; AP_MATMUL_MFMA4 (read once per process) forces either, so each is run
+    in a child process on shapes the default rule would give to the other."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import sys, numpy as np, torch
+sys.path[:0] = [%r, %r, %r]
+import oracle, any_precision_ext as ext
+from _util import assert_close_gemv, layer_to_gpu, make
+from any_precision_amd import synth
+for N, K in ((40, 2080), (2056, 1024), (9, 11008)):
+    L = make(N, K, seed=N)
+    q, luts = layer_to_gpu(L)
+    for b in (3, 6, 8):
+        for M in (2, 3, 4):
+            print(f"forced kernel N={N} K={K} b={b} M={M}", flush=True)
+            x = synth.make_x(M, K, seed=M)
+            got = ext.matmul_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
+print("ok")
+"""
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = code % (root, os.path.join(root, "any-precision-llm_amd"), os.path.join(root, "tests"))
+    for mode in ("0", "2"):
+        env = dict(os.environ, AP_MATMUL_MFMA4=mode)
+        res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=280)
+        assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (mode, res.stdout[-2000:], res.stderr[-2000:])
