@@ -30,7 +30,7 @@ def test_ragged_shapes_all_bits(ext, oracle, N, K):
     L = make(N, K, seed=N + K)
     q, luts = layer_to_gpu(L)
     for b in range(3, 9):
-        for M in (1, 9, 16, 33, 128):
+        for M in (1, 9, 16, 20, 32, 33, 128):
             print(f"gemm N={N} K={K} b={b} M={M}", flush=True)
             x, xg = _x(M, K, seed=M)
             got = ext.gemm_kbit(xg, q, luts[b], b)
