@@ -284,6 +284,20 @@ def main():
                     row[f"us_M{M}"] = round(time_graph(lambda st: launch(N, K, b, st, M, fn), 24), 2)
                 batch_table.append(row)
 
+    # ---- what this box gives a trivial kernel, in this run: a plain device copy (read 512 MiB + write
+    # 512 MiB per launch) and an elementwise op on one element (the fixed cost of a graph node)
+    machine = None
+    if not args.only_step and not args.eager:
+        src = torch.empty(128 << 20, dtype=torch.int32, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        us_copy = time_graph(lambda st: dst.copy_(src), 4)
+        one = torch.zeros(1, device="cuda")
+        us_node = time_graph(lambda st: one.add_(1.0), 200)
+        machine = {"copy_GBps": round(2 * src.numel() * 4 / us_copy / 1e3, 1), "copy_bytes": 2 * src.numel() * 4,
+                   "graph_node_us": round(us_node, 3),
+                   "note": "torch copy of 512 MiB (read + write) and a 1-element add, both as HIP-graph nodes"}
+        del src, dst
+
     roofline = None
     if table:
         dom = max(table, key=lambda r: r["us"] * r["count_in_step"])
@@ -363,7 +377,8 @@ def main():
                    "weight_sets_per_shape": {f"{N}x{K}": P.sets for (N, K), P in pools.items()},
                    "bytes_per_step": step_bytes,
                    "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu, "grouped_launches": grouped, "layers": table,
+        "roofline": roofline, "cpu_baseline": cpu, "grouped_launches": grouped, "machine_reference": machine,
+        "layers": table,
         "dequant_kbit": dequant_table, "batch_us": batch_table,
     }
     if args.table and table:
