@@ -245,7 +245,7 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
     GemvGeometry geo;
     GemvMembers mem = {};
     const int rc = gemv_geometry(M, N, count, K, w_bits, &geo, &mem);
-    if (rc != AP_OK) return rc;
+    if (rc != AP_OK && rc != AP_ELIMIT) return rc;
     if (!aligned16(x)) return AP_EALIGN;
     for (int g = 0; g < count; g++) {
         if (!aligned16(qweight[g]) || !aligned16(lut[g])) return AP_EALIGN;
@@ -254,6 +254,15 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
         mem.out[g] = out[g];
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (rc == AP_ELIMIT) {
+        // a row longer than one workgroup of the dot-product kernel covers (65536 elements at M <= 2,
+        // 32768 beyond): the MFMA kernel walks rows of any length
+        for (int g = 0; g < count; g++) {
+            const int r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
+            if (r != AP_OK) return r;
+        }
+        return AP_OK;
+    }
     // 3 and 4 activation rows at up to 5 bits on linears with enough rows to fill the chip (8 per
     // workgroup): the 4x4x4 matrix-core kernel, 10-35 % faster there than the dot-product kernel, whose
     // cost grows with M.  It serves one linear per launch.

@@ -212,3 +212,23 @@ print("ok")
         env = dict(os.environ, AP_MATMUL_MFMA4=mode)
         res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=280)
         assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (mode, res.stdout[-2000:], res.stderr[-2000:])
+
+
+def test_rows_longer_than_a_workgroup_covers(ext):
+    """K beyond what one workgroup of the dot-product kernel spans (65536 at M <= 2, 32768 at 3..4):
+    the entry point falls back to the MFMA kernel.  Reference: fp32 matmul of the dequantised weight."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    for K, Ms in ((66560, (1, 2)), (40960, (3, 4, 8))):
+        N = 24
+        q = torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda", generator=gen)
+        for b in (3, 8):
+            lut = torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02, dim=1).values.half()
+            w = ext.dequant_kbit(q, lut, b).double()
+            for M in Ms:
+                print(f"long rows K={K} b={b} M={M}", flush=True)
+                x = torch.randn((M, K), device="cuda", generator=gen).half()
+                want = x.double() @ w.T
+                got = ext.matmul_kbit(x, q, lut, b).double()
+                assert (got - want).norm() <= 1e-2 * want.norm()
+                assert (got - want).abs().max() <= 1e-2 * want.abs().max()
