@@ -6,7 +6,7 @@ Hugging Face loop (demo.py:59-80), which at batch 1 is bound by Python and launc
 not by the kernels.  Here one decode step -- embedding, 32 x (norm, q/k/v GEMV, rotary,
 cache write, attention over a static cache, o GEMV, norm, gate/up GEMV, SiLU, down GEMV),
 final norm, head, argmax, position increment -- is recorded once per precision and replayed
-per token: no host work between tokens.  Only the seven linears per layer are this
+per token: no host work between tokens, 19 kernel launches per layer.  Only the seven linears per layer are this
 library's kernels (q/k/v and gate/up as one grouped launch each); everything else is stock
 PyTorch ops, as in the reference.
 
@@ -23,9 +23,10 @@ import torch.nn.functional as F
 from .linear import forward_group
 
 
-def _rotate_half(x):
-    h = x.shape[-1] // 2
-    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+def _rope(x, cos, sin_signed):
+    """Rotary embedding of x [T, heads, hd] in three kernels: x * cos + rotate_half(x) * sin, with
+    rotate_half(x) * sin written as roll(x, hd / 2) * (sin with its first half negated)."""
+    return torch.addcmul(torch.roll(x, x.shape[-1] // 2, dims=-1) * sin_signed, x, cos)
 
 
 class GraphDecoder:
@@ -58,11 +59,18 @@ class GraphDecoder:
         inv = 1.0 / (theta ** (torch.arange(0, self.hd, 2, device=dev, dtype=torch.float32) / self.hd))
         ang = torch.outer(torch.arange(max_len, device=dev, dtype=torch.float32), inv)
         ang = torch.cat((ang, ang), dim=-1)
-        self.cos, self.sin = ang.cos().to(torch.float16), ang.sin().to(torch.float16)     # [max_len, hd]
+        self.cos = ang.cos().to(torch.float16)                                              # [max_len, hd]
+        sin = ang.sin()
+        self.sin_signed = torch.cat((-sin[:, :self.hd // 2], sin[:, self.hd // 2:]), dim=-1).to(torch.float16)
+        # additive attention mask, one row per position: 0 up to and including it, -inf beyond
+        self.mask = torch.zeros((max_len, max_len), dtype=torch.float16, device=dev)
+        self.mask.masked_fill_(torch.arange(max_len, device=dev)[None, :] > torch.arange(max_len, device=dev)[:, None],
+                               float("-inf"))
         L = len(self.layers)
         self.kcache = torch.zeros((L, self.nkv, max_len, self.hd), dtype=torch.float16, device=dev)
         self.vcache = torch.zeros_like(self.kcache)
-        self.arange = torch.arange(max_len, device=dev)
+        self.head_scale = torch.cat((torch.full((self.nh,), 1.0 / math.sqrt(self.hd)), torch.ones(self.nkv))) \
+            .to(torch.float16).to(dev).view(1, self.nh + self.nkv, 1)
         # state the captured step reads and advances
         self.tok = torch.zeros((1,), dtype=torch.long, device=dev)
         self.pos = torch.zeros((1,), dtype=torch.long, device=dev)
@@ -72,45 +80,50 @@ class GraphDecoder:
         self.stream = torch.cuda.Stream(device=dev)
 
     # ------------------------------------------------------------------ the network
-    def _group(self, modules, x, precision):
-        if self.group_launches:
-            return forward_group(modules, x, precision)
-        return [m(x, precision=precision) for m in modules]
-
     def _norm(self, x, w):
         return F.rms_norm(x, (x.shape[-1],), w, self.eps)
 
-    def _layer(self, li, h, pos_idx, cos, sin, mask, precision):
-        """h [T, H]; pos_idx [T] cache rows of these tokens; mask [T, max_len] additive."""
+    def _layer(self, li, h, pos_idx, cos, sin_signed, mask, precision):
+        """h [T, H]; pos_idx [T] cache rows of these tokens; mask [nkv, g * T, max_len] additive, fp16.
+        Kernel launches per layer and token: 2 norms, 5 for the linears (q/k/v and gate/up grouped),
+        3 rotary, 2 cache writes, 3 attention, 2 residual adds, 2 for SiLU * up."""
         layer = self.layers[li]
         T = h.shape[0]
+        att = layer.self_attn
+        nq, nk = self.nh * self.hd, self.nkv * self.hd
         x = self._norm(h, layer.input_layernorm.weight)
-        att_in = layer.self_attn
-        q, k, v = self._group((att_in.q_proj, att_in.k_proj, att_in.v_proj), x, precision)
-        q, k, v = q.view(T, self.nh, self.hd), k.view(T, self.nkv, self.hd), v.view(T, self.nkv, self.hd)
-        q = q * cos + _rotate_half(q) * sin
-        k = k * cos + _rotate_half(k) * sin
-        self.kcache[li].index_copy_(1, pos_idx, k.transpose(0, 1))
+        if self.group_launches:
+            qkv = forward_group((att.q_proj, att.k_proj, att.v_proj), x, precision, concat=True)       # [T, nq + 2 nk]
+        else:
+            qkv = torch.cat([m(x, precision=precision) for m in (att.q_proj, att.k_proj, att.v_proj)], dim=-1)
+        qk = _rope(qkv[:, :nq + nk].view(T, self.nh + self.nkv, self.hd), cos, sin_signed)             # q scaled by 1/sqrt(hd)
+        v = qkv[:, nq + nk:].view(T, self.nkv, self.hd)
+        self.kcache[li].index_copy_(1, pos_idx, qk[:, self.nh:].transpose(0, 1))
         self.vcache[li].index_copy_(1, pos_idx, v.transpose(0, 1))
         g = self.nh // self.nkv
-        qh = q.transpose(0, 1).reshape(self.nkv, g * T, self.hd)                        # [nkv, g*T, hd]
-        scores = torch.bmm(qh, self.kcache[li].transpose(1, 2)).float() / math.sqrt(self.hd)   # [nkv, g*T, max_len]
-        scores = scores.view(self.nkv, g, T, self.max_len) + mask
-        probs = torch.softmax(scores, dim=-1).to(torch.float16).view(self.nkv, g * T, self.max_len)
-        att = torch.bmm(probs, self.vcache[li]).view(self.nh, T, self.hd).transpose(0, 1).reshape(T, self.nh * self.hd)
-        h = h + layer.self_attn.o_proj(att, precision=precision)
+        qh = qk[:, :self.nh].transpose(0, 1).reshape(self.nkv, g * T, self.hd)                         # [nkv, g*T, hd]
+        scores = torch.baddbmm(mask, qh, self.kcache[li].transpose(1, 2))                              # [nkv, g*T, max_len]
+        probs = torch.softmax(scores, dim=-1)
+        ctx = torch.bmm(probs, self.vcache[li]).view(self.nh, T, self.hd).transpose(0, 1).reshape(T, nq)
+        h = h + att.o_proj(ctx, precision=precision)
         x = self._norm(h, layer.post_attention_layernorm.weight)
-        gate, up = self._group((layer.mlp.gate_proj, layer.mlp.up_proj), x, precision)
+        if self.group_launches:
+            gate, up = forward_group((layer.mlp.gate_proj, layer.mlp.up_proj), x, precision)
+        else:
+            gate, up = layer.mlp.gate_proj(x, precision=precision), layer.mlp.up_proj(x, precision=precision)
         return h + layer.mlp.down_proj(F.silu(gate) * up, precision=precision)
 
     def _forward(self, tokens, pos_idx, precision):
         """tokens [T], pos_idx [T] (device tensors) -> logits of the last token [1, vocab]."""
+        T = tokens.shape[0]
         h = self.embed.index_select(0, tokens)
-        cos = self.cos.index_select(0, pos_idx).unsqueeze(1)
-        sin = self.sin.index_select(0, pos_idx).unsqueeze(1)
-        mask = torch.where(self.arange.unsqueeze(0) > pos_idx.unsqueeze(1), float("-inf"), 0.0)   # [T, max_len] fp32
+        # per-head rotary factors [T, nh + nkv, hd]; the query heads carry the 1/sqrt(hd) of the attention
+        cos = self.cos.index_select(0, pos_idx).unsqueeze(1) * self.head_scale
+        sin_signed = self.sin_signed.index_select(0, pos_idx).unsqueeze(1) * self.head_scale
+        g = self.nh // self.nkv
+        mask = self.mask.index_select(0, pos_idx).repeat(g, 1).unsqueeze(0).expand(self.nkv, g * T, self.max_len)
         for li in range(len(self.layers)):
-            h = self._layer(li, h, pos_idx, cos, sin, mask, precision)
+            h = self._layer(li, h, pos_idx, cos, sin_signed, mask, precision)
         h = self._norm(h[-1:], self.final_norm)
         return F.linear(h, self.head)
 

@@ -25,21 +25,27 @@ except ModuleNotFoundError:
 FUSED_GEMM_ROWS = min(32, GEMM_MAX_M)
 
 
-def forward_group(modules, x, precision=None):
+def forward_group(modules, x, precision=None, concat=False):
     """``[m(x, precision=precision) for m in modules]`` for linears that share their input (the
-    q/k/v or gate/up projections of a decoder layer).  Up to 4 activation rows and 4 modules
-    the GEMVs go out as ONE launch; otherwise module by module.  The reference has no
-    counterpart (its ``fuse_layers`` is a stub, AnyPrecisionForCausalLM.py:168-172)."""
+    q/k/v or gate/up projections of a decoder layer); with ``concat`` the results joined along
+    the last dimension.  Up to 4 activation rows and 4 modules the GEMVs go out as ONE launch;
+    otherwise module by module.  The reference has no counterpart (its ``fuse_layers`` is a
+    stub, AnyPrecisionForCausalLM.py:168-172)."""
     rows = x.numel() // x.shape[-1]
     w_bits = modules[0].precision if precision is None else precision
     if rows > 4 or not 2 <= len(modules) <= 4 or not x.is_contiguous() or any(
             m.in_features != modules[0].in_features for m in modules):
-        return [m(x, precision=w_bits) for m in modules]
-    outs = matmul_kbit_group(x, [m.qweight for m in modules], [m._buffers[f"lut{w_bits}"] for m in modules], w_bits)
-    for m, o in zip(modules, outs):
+        outs = [m(x, precision=w_bits) for m in modules]
+        return torch.cat(outs, dim=-1) if concat else outs
+    has_bias = any(m.bias is not None for m in modules)
+    res = matmul_kbit_group(x, [m.qweight for m in modules], [m._buffers[f"lut{w_bits}"] for m in modules], w_bits,
+                            concat=concat and not has_bias)
+    if not has_bias:
+        return res
+    for m, o in zip(modules, res):
         if m.bias is not None:
             o += m.bias
-    return outs
+    return torch.cat(res, dim=-1) if concat else res
 
 
 class AnyPrecisionLinear(nn.Module):

@@ -86,10 +86,12 @@ def matmul_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_b
     return out
 
 
-def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int):
+def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int, concat: bool = False):
     """``[matmul_kbit(in_, q, t, w_bits) for q, t in zip(qweights, luts)]`` in one launch: up to
     GROUP_MAX linears that share the input and the bit-width (q/k/v, gate/up).  No counterpart in
-    the reference; results equal the separate calls bit for bit."""
+    the reference; results equal the separate calls bit for bit.  ``concat=True`` returns the
+    results joined along the last dimension as one tensor (for a single activation row they are
+    written side by side into one allocation; otherwise joined with ``torch.cat``)."""
     if len(qweights) != len(luts) or not 1 <= len(qweights) <= _capi.GROUP_MAX:
         raise ValueError(f"matmul_kbit_group: need 1..{_capi.GROUP_MAX} (qweight, lut) pairs")
     shapes = [_check_weight(q, t, w_bits, "matmul_kbit_group") for q, t in zip(qweights, luts)]
@@ -108,11 +110,18 @@ def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int):
     if not in_.is_contiguous():
         raise ValueError("matmul_kbit_group: input must be contiguous")
     with torch.cuda.device(in_.device):
-        outs = [torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device) for N, _ in shapes]
+        joint = None
+        if concat and M == 1:
+            joint = torch.empty(in_.shape[:-1] + (sum(N for N, _ in shapes),), dtype=torch.float16, device=in_.device)
+            outs = list(torch.split(joint, [N for N, _ in shapes], dim=-1))       # one row: every part is dense
+        else:
+            outs = [torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device) for N, _ in shapes]
         rc = _capi.matmul_group(in_.data_ptr(), [q.data_ptr() for q in qweights], [t.data_ptr() for t in luts],
                                 [o.data_ptr() for o in outs], [N for N, _ in shapes], M, K, w_bits,
                                 torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "matmul_kbit_group")
+    if concat:
+        return joint if joint is not None else torch.cat(outs, dim=-1)
     return outs
 
 
