@@ -232,3 +232,22 @@ def test_rows_longer_than_a_workgroup_covers(ext):
                 got = ext.matmul_kbit(x, q, lut, b).double()
                 assert (got - want).norm() <= 1e-2 * want.norm()
                 assert (got - want).abs().max() <= 1e-2 * want.abs().max()
+
+
+def test_denormal_table_entries_are_not_flushed(ext, oracle):
+    """Tables whose entries are fp16 denormals (|w| ~ 1e-5 < 6.1e-5): every kernel must multiply them
+    as they are (fp16 products, fp32 accumulate); flushing them to zero would return zeros."""
+    L = make(64, 4096, seed=3)
+    q, _ = layer_to_gpu(L)
+    for b in (3, 5, 8):
+        lut = (L.luts[b].astype(np.float32) * 5e-4).astype(np.float16)
+        assert 0 < np.abs(lut).max() < 6.1e-5
+        lg = torch.from_numpy(lut).cuda()
+        for M, fn in ((1, ext.matmul_kbit), (2, ext.matmul_kbit), (4, ext.matmul_kbit), (8, ext.matmul_kbit),
+                      (24, ext.gemm_kbit)):
+            print(f"denormal tables b={b} M={M}", flush=True)
+            x, xg = _x(M, L.K, seed=M)
+            got = fn(xg, q, lg, b)
+            _, want = oracle.matmul_kbit(x, L.qweight, lut, b, return_f64=True)
+            assert np.abs(want).max() > 5e-6
+            assert_close_gemv(got, want, f"denormal tables b={b} M={M}")
