@@ -22,7 +22,7 @@ struct Tuning {
     int dequant_blocks_per_cu;
     int mfma_from_rows;     // ap_matmul_kbit uses the MFMA kernel from this many activation rows on
     int force_gemm_split;   // > 0: K-split waves per workgroup of the fused GEMM
-    int mfma4_mode;         // 4x4x4 matrix-core kernel: 0 never, 1 for 3..4 rows at up to 5 bits, 2 for 2..4 rows always
+    int mfma4_mode;         // 4x4x4 matrix-core kernel: 0 never, 1 where it pays (3..4 rows), 2 for 2..4 rows always
     int force_gemv4_groups; // > 0: word groups per wave of that kernel
 };
 
@@ -263,15 +263,16 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
         }
         return AP_OK;
     }
-    // 3 and 4 activation rows at up to 5 bits on linears with enough rows to fill the chip (8 per
-    // workgroup): the 4x4x4 matrix-core kernel, 10-35 % faster there than the dot-product kernel, whose
-    // cost grows with M.  It serves one linear per launch.
+    // 3 and 4 activation rows on linears with enough rows to fill the chip (8 per workgroup): the
+    // 4x4x4 matrix-core kernel, whose cost does not grow with M -- at up to 5 bits, and for 4 rows at
+    // every bit-width while a row fits one word group per lane (K <= 8192).  10-40 % faster there
+    // than the dot-product kernel.  It serves one linear per launch.
     const int m4 = tuning().mfma4_mode;
     const bool fits4 = (K >> 5) <= 16 * 4 * kGemv4MaxSeg;  // at most 4 word groups per wave, 16 waves
     long long rows = 0;
     for (int g = 0; g < count; g++) rows += N[g];
-    if (fits4 && ((m4 == 1 && M >= 3 && M <= 4 && w_bits <= 5 && rows >= 2048LL * count) ||
-                  (m4 == 2 && M >= 2 && M <= 4))) {
+    const bool pays4 = (M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192));
+    if (fits4 && ((m4 == 1 && pays4 && rows >= 2048LL * count) || (m4 == 2 && M >= 2 && M <= 4))) {
         for (int g = 0; g < count; g++) {
             const int r = run_gemv4(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
             if (r != AP_OK) return r;

@@ -48,7 +48,10 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     constexpr int MAXS = THREADS / kWave;
     constexpr int MR = 4 * MG;  // activation rows computed (rows past M repeat row M-1 and are not stored)
     constexpr int ROWS = 4 * RQ;
-    __shared__ __attribute__((aligned(16))) half_t tables[ROWS][NC];
+    // plain tables at every bit-width: pair tables (two weights per entry, as in the dot-product
+    // kernel) measured equal or slower here, the permuted activations cost what the packing saves
+    constexpr int TB = 2 << BITS;
+    __shared__ __attribute__((aligned(16))) uint8_t tables[ROWS][TB];
     __shared__ float partial[MAXS][ROWS][MR];  // [wave][weight row][activation row]
 
     const int lane = threadIdx.x;
@@ -92,6 +95,7 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
             for (int p = 0; p < BITS; p++) q[rq][g][p] = __builtin_nontemporal_load(wrow + p * plane_stride + w);
         }
     }
+    // X[mg][g][j]: the eight activations of byte group j of this lane's word, row 4 mg + qi
     u32x4 X[MG][G][4];
 #pragma unroll
     for (int mg = 0; mg < MG; mg++) {
@@ -102,40 +106,42 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
             for (int j = 0; j < 4; j++)
                 X[mg][g][j] = *reinterpret_cast<const u32x4 *>(xrow + group_base(wl[g], j, K));
     }
-    // words past the row end: all four lanes of their block are past it, so zero activations
-    // silence the whole block
+    // words past the row end (last wave of a row only): all four lanes of their block are past it,
+    // so zero activations silence the whole block
+    if ((s * G + G) * 16 > W) {
 #pragma unroll
-    for (int mg = 0; mg < MG; mg++)
+        for (int mg = 0; mg < MG; mg++)
 #pragma unroll
-        for (int g = 0; g < G; g++)
+            for (int g = 0; g < G; g++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (!live[g]) X[mg][g][j] = u32x4{0u, 0u, 0u, 0u};
+                for (int j = 0; j < 4; j++)
+                    if (!live[g]) X[mg][g][j] = u32x4{0u, 0u, 0u, 0u};
+    }
 
 #pragma unroll
     for (int r = 0; r < ROWS; r++)
-        if (s == (r & pmask)) lut_stage<BITS>(t[r], tables[r], lane);
+        if (s == (r & pmask)) lut_stage<BITS>(t[r], reinterpret_cast<half_t *>(tables[r]), lane);
     if (S > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
 
     // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
-    typedef __attribute__((address_space(3))) half_t lds_half_t;
-    const uint32_t tab_base0 = (uint32_t)(uintptr_t)((lds_half_t *)&tables[0][0]) + (uint32_t)qi * (NC * 2);
+    typedef __attribute__((address_space(3))) uint8_t lds_byte_t;
+    const uint32_t tab_base0 = (uint32_t)(uintptr_t)((lds_byte_t *)&tables[0][0]) + (uint32_t)qi * TB;
 
     static_for<RQ>([&](auto rq_c) {
     constexpr int rq = decltype(rq_c)::value;
-    const uint32_t tab_base = tab_base0 + rq * 4 * NC * 2;
+    const uint32_t tab_base = tab_base0 + rq * 4 * TB;
     f32x4_t acc[MG];
 #pragma unroll
     for (int mg = 0; mg < MG; mg++) acc[mg] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     static_for<G>([&](auto g_c) {
         constexpr int g = decltype(g_c)::value;
-        // index bytes hold the byte offset into the table (index * 2) where that fits a byte
-        constexpr int PRE = BITS <= 7 ? 1 : 0;
-        uint32_t idx[8];
         uint32_t qq[BITS];
 #pragma unroll
         for (int p = 0; p < BITS; p++) qq[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(take, (int)q[rq][g][p]);
+        // index bytes hold the byte offset into the table (index * 2) where that fits a byte
+        constexpr int PRE = BITS <= 7 ? 1 : 0;
+        uint32_t idx[8];
         planes_to_indices<BITS, PRE>(qq, idx);
         static_for<4>([&](auto j_c) {
             constexpr int j = decltype(j_c)::value, c = 3 - j;
@@ -166,24 +172,33 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
         });
     });
 
-    // Sum over the 16 blocks, i.e. over the lanes with the same l % 4: two shifted adds within
-    // each 16-lane row (sums in its lanes 12..15), then two half/quarter swaps across the four
-    // rows (every row holds the total).  Lanes 12..15 of row 0 park it in LDS for the S waves.
+    // Sum over the 16 blocks, i.e. over the lanes with the same l % 4.  Two shifted adds within each
+    // 16-lane row leave the row's sums in its lanes 12..15; the four rows are then folded with
+    // half / quarter swaps BETWEEN the four accumulators, so that one add serves two of them:
+    // afterwards row r of `u` holds the total of accumulator kOrder[r].
 #pragma unroll
-    for (int mg = 0; mg < MG; mg++)
+    for (int mg = 0; mg < MG; mg++) {
+        uint32_t v[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            float v = acc[mg][i];
-            v = dpp_add<0x114>(v);  // row_shr:4
-            v = dpp_add<0x118>(v);  // row_shr:8
-            const uint32_t u = __builtin_bit_cast(uint32_t, v);
-            const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // rows 2,3 <-> rows 0,1
-            v = __builtin_bit_cast(float, (uint32_t)h[0]) + __builtin_bit_cast(float, (uint32_t)h[1]);
-            const uint32_t u2 = __builtin_bit_cast(uint32_t, v);
-            const auto qd = __builtin_amdgcn_permlane16_swap(u2, u2, false, false);  // odd rows <-> even rows
-            v = __builtin_bit_cast(float, (uint32_t)qd[0]) + __builtin_bit_cast(float, (uint32_t)qd[1]);
-            if (lane >= 12 && lane < 16) partial[s][4 * rq + qi][mg * 4 + i] = v;
+            float f = acc[mg][i];
+            f = dpp_add<0x114>(f);  // row_shr:4
+            f = dpp_add<0x118>(f);  // row_shr:8
+            v[i] = __builtin_bit_cast(uint32_t, f);
         }
+        auto fold32 = [](uint32_t a, uint32_t b) {  // rows 0,1: a(0+2, 1+3); rows 2,3: b(0+2, 1+3)
+            const auto h = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+            return __builtin_bit_cast(float, (uint32_t)h[0]) + __builtin_bit_cast(float, (uint32_t)h[1]);
+        };
+        const float t01 = fold32(v[0], v[1]), t23 = fold32(v[2], v[3]);
+        const auto qd = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(uint32_t, t01), __builtin_bit_cast(uint32_t, t23),
+                                                         false, false);
+        const float u = __builtin_bit_cast(float, (uint32_t)qd[0]) + __builtin_bit_cast(float, (uint32_t)qd[1]);
+        // rows 0..3 of u: totals of accumulators 0, 2, 1, 3
+        const int r16 = lane >> 4;
+        const int which = ((r16 & 1) << 1) | (r16 >> 1);
+        if ((lane & 15) >= 12) partial[s][4 * rq + qi][mg * 4 + which] = u;
+    }
     });
     __syncthreads();
     for (int o = s * kWave + lane; o < ROWS * MR; o += S * kWave) {
