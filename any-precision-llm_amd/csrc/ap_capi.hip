@@ -22,7 +22,7 @@ struct Tuning {
     int dequant_blocks_per_cu;
     int mfma_from_rows;     // ap_matmul_kbit uses the MFMA kernel from this many activation rows on
     int force_gemm_split;   // > 0: K-split waves per workgroup of the fused GEMM
-    int mfma4_mode;         // 4x4x4 matrix-core kernel: 0 never, 1 where it pays (3..4 rows), 2 for 2..4 rows always
+    int mfma4_mode;         // 4x4x4 matrix-core kernel: 0 never, 1 where it pays, 2 for 2..8 rows wherever it fits
     int force_gemv4_groups; // > 0: word groups per wave of that kernel
 };
 
@@ -193,19 +193,28 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
 int run_gemv4(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
               int w_bits, hipStream_t st) {
     Gemv4Geometry geo;
-    if (M > 4) return AP_EBATCH;
-    geo.mg = 1;
-    geo.rq = 2;
-    geo.grid = (N + 4 * geo.rq - 1) / (4 * geo.rq);
+    if (M > 8) return AP_EBATCH;
     const int W = K >> 5;
-    // one word group per wave (with two row quads: 64 weights per lane, as in the dot-product kernel)
-    // unless the row is so long that a workgroup could not hold its waves
-    int G = tuning().force_gemv4_groups > 0 ? tuning().force_gemv4_groups : 1;
-    if (G != 1 && G != 2 && G != 4) G = 1;
-    while (G < 4 && (W + 16 * G - 1) / (16 * G) > kGemv4MaxSeg) G *= 2;
-    geo.G = G;
-    geo.S = (W + 16 * G - 1) / (16 * G);
-    if (geo.S > kGemv4MaxSeg) return AP_ELIMIT;
+    if (M > 4) {
+        // two groups of four activation rows: four row quads per workgroup, one word group per wave
+        geo.mg = 2;
+        geo.rq = 4;
+        geo.G = 1;
+        geo.S = (W + 15) / 16;
+        if (geo.S > kGemv4MaxSegTwo) return AP_ELIMIT;
+    } else {
+        geo.mg = 1;
+        geo.rq = 2;
+        // one word group per wave (with two row quads: 64 weights per lane, as in the dot-product kernel)
+        // unless the row is so long that a workgroup could not hold its waves
+        int G = tuning().force_gemv4_groups > 0 ? tuning().force_gemv4_groups : 1;
+        if (G != 1 && G != 2 && G != 4) G = 1;
+        while (G < 4 && (W + 16 * G - 1) / (16 * G) > kGemv4MaxSeg) G *= 2;
+        geo.G = G;
+        geo.S = (W + 16 * G - 1) / (16 * G);
+        if (geo.S > kGemv4MaxSeg) return AP_ELIMIT;
+    }
+    geo.grid = (N + 4 * geo.rq - 1) / (4 * geo.rq);
     switch (w_bits) {
         case 3: launch_gemv4<3>(geo, x, qweight, lut, out, M, N, K, st); break;
         case 4: launch_gemv4<4>(geo, x, qweight, lut, out, M, N, K, st); break;
@@ -263,18 +272,35 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
         }
         return AP_OK;
     }
-    // 3 and 4 activation rows on linears with enough rows to fill the chip (8 per workgroup): the
-    // 4x4x4 matrix-core kernel, whose cost does not grow with M -- at up to 5 bits, and for 4 rows at
-    // every bit-width while a row fits one word group per lane (K <= 8192).  10-40 % faster there
-    // than the dot-product kernel.  It serves one linear per launch.
+    // The 4x4x4 matrix-core kernel, whose cost per weight does not grow with M, where it measured
+    // faster than both other kernels (it serves one linear per launch):
+    //  - 3 and 4 activation rows on linears with enough rows to fill the chip (8 per workgroup), at up
+    //    to 5 bits, and for 4 rows at every bit-width while a row fits one word group per lane
+    //    (K <= 8192): 10-40 % faster than the dot-product kernel;
+    //  - 5..8 activation rows on wide linears (16 rows per workgroup) with rows of 3072..4096 elements
+    //    (5..8 waves per workgroup): 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and longer
+    //    rows and narrower linears measured slower.
     const int m4 = tuning().mfma4_mode;
-    const bool fits4 = (K >> 5) <= 16 * 4 * kGemv4MaxSeg;  // at most 4 word groups per wave, 16 waves
     long long rows = 0;
     for (int g = 0; g < count; g++) rows += N[g];
-    const bool pays4 = (M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192));
-    if (fits4 && ((m4 == 1 && pays4 && rows >= 2048LL * count) || (m4 == 2 && M >= 2 && M <= 4))) {
+    auto use4 = [&](int n) {
+        const int W = K >> 5;
+        if (m4 == 0 || M < 2 || M > 8) return false;
+        if (M <= 4) {  // decided for the group as a whole, by its mean row count
+            if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
+            if (m4 >= 2) return true;
+            return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192))) && rows >= 2048LL * count;
+        }
+        if (W > 16 * kGemv4MaxSegTwo) return false;
+        if (m4 >= 2) return true;
+        return K >= 3072 && n >= 10240;  // per member; the others go to the MFMA kernel
+    };
+    bool any4 = false;
+    for (int g = 0; g < count; g++) any4 |= use4(N[g]);
+    if (any4) {
         for (int g = 0; g < count; g++) {
-            const int r = run_gemv4(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
+            const int r = use4(N[g]) ? run_gemv4(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st)
+                                     : run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
             if (r != AP_OK) return r;
         }
         return AP_OK;

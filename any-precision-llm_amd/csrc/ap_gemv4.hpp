@@ -1,5 +1,6 @@
 // Bitplane skinny GEMM for gfx950 on the 4x4x4 matrix cores, up to 4 MG activation rows
-// (used for 3 and 4 rows, where it beats both other kernels at up to 6 bits):
+// (used for 3 and 4 rows, and for 5..8 rows on wide linears with rows of about 4096 elements,
+// where it beats both other kernels):
 //     out[m,n] = sum_k x[m,k] * lut[n, index_b(n,k)]      (fp16 operands, fp32 accumulate)
 //
 // Same operator as the reference's matmul_kbit_32 with multi_row (any_precision/modules/

@@ -6,17 +6,18 @@
 
 namespace ap {
 
-constexpr int kGemv4MaxSeg = 16;  // waves per workgroup
+constexpr int kGemv4MaxSeg = 16;      // waves per workgroup, up to 4 activation rows
+constexpr int kGemv4MaxSegTwo = 8;    // waves per workgroup, 5..8 activation rows
 
 struct Gemv4Geometry {
-    int mg;    // groups of four activation rows (1: only that is instantiated)
-    int G;     // word groups (16 words of each of 4 rows) per wave: 1, 2 or 4
+    int mg;    // groups of four activation rows: 1 or 2
+    int G;     // word groups (16 words of each of 4 rows) per wave: 1, 2 or 4 (mg = 2: 1 only)
     int S;     // waves per workgroup
-    int rq;    // row quads per workgroup (2: only that is instantiated)
+    int rq;    // row quads per workgroup: 2 with mg = 1, 4 with mg = 2 (only those are instantiated)
     int grid;  // workgroups = ceil(N / (4 rq))
 };
 
-// Launches gemv4_kbit_kernel<BITS, 1, geo.G, 2, *> on `stream`.  1 <= M <= 4.
+// Launches gemv4_kbit_kernel<BITS, 1, geo.G, 2, *> (1 <= M <= 4) or <BITS, 2, 1, 4, *> (5 <= M <= 8) on `stream`.
 template <int BITS>
 void launch_gemv4(const Gemv4Geometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                   uint16_t *out, int M, int N, int K, hipStream_t stream);

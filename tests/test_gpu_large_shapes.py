@@ -46,3 +46,24 @@ def test_llama70b_mlp_shapes(N, K):
             assert (got - want).norm() <= REL_TOL * want.norm(), f"{fn.__name__} M={M} b={b}"
             assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"{fn.__name__} M={M} b={b}"
         del want_w
+
+
+def test_llama3_8b_mlp_shape_at_every_batch_up_to_eight():
+    """14336 x 4096 at M = 1..8 under the default routing: the dot-product kernel (1, 2 and part of
+    3), the 4x4x4 matrix-core kernel with one (3, 4) and two (5..8) groups of activation rows."""
+    import any_precision_ext as ext
+    N, K = 14336, 4096
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    q = torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda", generator=gen)
+    for b in (3, 4, 5, 6, 7, 8):
+        lut = torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02, dim=1).values.half()
+        want_w = torch.gather(lut, 1, torch_indices(q, b)).double()
+        for M in range(1, 9):
+            print(f"llama3 mlp b={b} M={M}", flush=True)
+            x = torch.randn((M, K), device="cuda", generator=gen).half()
+            want = x.double() @ want_w.T
+            got = ext.matmul_kbit(x, q, lut, b).double()
+            assert (got - want).norm() <= REL_TOL * want.norm(), f"M={M} b={b}"
+            assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"M={M} b={b}"
+        del want_w

@@ -198,7 +198,7 @@ for N, K in ((40, 2080), (2056, 1024), (9, 11008)):
     L = make(N, K, seed=N)
     q, luts = layer_to_gpu(L)
     for b in (3, 6, 8):
-        for M in (2, 3, 4):
+        for M in (2, 3, 4, 5, 7, 8):
             print(f"forced kernel N={N} K={K} b={b} M={M}", flush=True)
             x = synth.make_x(M, K, seed=M)
             got = ext.matmul_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
