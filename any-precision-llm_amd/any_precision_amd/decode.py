@@ -67,8 +67,10 @@ class GraphDecoder:
         self.mask.masked_fill_(torch.arange(max_len, device=dev)[None, :] > torch.arange(max_len, device=dev)[:, None],
                                float("-inf"))
         L = len(self.layers)
-        self.kcache = torch.zeros((L, self.nkv, max_len, self.hd), dtype=torch.float16, device=dev)
-        self.vcache = torch.zeros_like(self.kcache)
+        # keys and values of a layer side by side (heads 0..nkv-1 keys, nkv..2nkv-1 values): one write per layer
+        self.kvcache = torch.zeros((L, 2 * self.nkv, max_len, self.hd), dtype=torch.float16, device=dev)
+        self.kcache = self.kvcache[:, :self.nkv]
+        self.vcache = self.kvcache[:, self.nkv:]
         self.head_scale = torch.cat((torch.full((self.nh,), 1.0 / math.sqrt(self.hd)), torch.ones(self.nkv))) \
             .to(torch.float16).to(dev).view(1, self.nh + self.nkv, 1)
         # state the captured step reads and advances
@@ -86,7 +88,8 @@ class GraphDecoder:
     def _layer(self, li, h, pos_idx, cos, sin_signed, mask, precision):
         """h [T, H]; pos_idx [T] cache rows of these tokens; mask [nkv, g * T, max_len] additive, fp16.
         Kernel launches per layer and token: 2 norms, 5 for the linears (q/k/v and gate/up grouped),
-        3 rotary, 2 cache writes, 3 attention, 2 residual adds, 2 for SiLU * up."""
+        3 rotary, 1 cache write, 4 attention (mask copy, scores, softmax, context), 2 residual adds,
+        2 for SiLU * up."""
         layer = self.layers[li]
         T = h.shape[0]
         att = layer.self_attn
@@ -96,12 +99,11 @@ class GraphDecoder:
             qkv = forward_group((att.q_proj, att.k_proj, att.v_proj), x, precision, concat=True)       # [T, nq + 2 nk]
         else:
             qkv = torch.cat([m(x, precision=precision) for m in (att.q_proj, att.k_proj, att.v_proj)], dim=-1)
-        qk = _rope(qkv[:, :nq + nk].view(T, self.nh + self.nkv, self.hd), cos, sin_signed)             # q scaled by 1/sqrt(hd)
-        v = qkv[:, nq + nk:].view(T, self.nkv, self.hd)
-        self.kcache[li].index_copy_(1, pos_idx, qk[:, self.nh:].transpose(0, 1))
-        self.vcache[li].index_copy_(1, pos_idx, v.transpose(0, 1))
+        # rotary over all heads at once: the value heads carry cos = 1, sin = 0; q comes out scaled by 1/sqrt(hd)
+        qkv = _rope(qkv.view(T, self.nh + 2 * self.nkv, self.hd), cos, sin_signed)
+        self.kvcache[li].index_copy_(1, pos_idx, qkv[:, self.nh:].transpose(0, 1))
         g = self.nh // self.nkv
-        qh = qk[:, :self.nh].transpose(0, 1).reshape(self.nkv, g * T, self.hd)                         # [nkv, g*T, hd]
+        qh = qkv[:, :self.nh].transpose(0, 1).reshape(self.nkv, g * T, self.hd)                        # [nkv, g*T, hd]
         scores = torch.baddbmm(mask, qh, self.kcache[li].transpose(1, 2))                              # [nkv, g*T, max_len]
         probs = torch.softmax(scores, dim=-1)
         ctx = torch.bmm(probs, self.vcache[li]).view(self.nh, T, self.hd).transpose(0, 1).reshape(T, nq)
@@ -117,9 +119,12 @@ class GraphDecoder:
         """tokens [T], pos_idx [T] (device tensors) -> logits of the last token [1, vocab]."""
         T = tokens.shape[0]
         h = self.embed.index_select(0, tokens)
-        # per-head rotary factors [T, nh + nkv, hd]; the query heads carry the 1/sqrt(hd) of the attention
+        # per-head rotary factors [T, nh + 2 nkv, hd]: the query heads carry the 1/sqrt(hd) of the attention,
+        # the value heads pass through (cos = 1, sin = 0)
         cos = self.cos.index_select(0, pos_idx).unsqueeze(1) * self.head_scale
         sin_signed = self.sin_signed.index_select(0, pos_idx).unsqueeze(1) * self.head_scale
+        cos = torch.cat((cos, cos.new_ones((T, self.nkv, self.hd))), dim=1)
+        sin_signed = torch.cat((sin_signed, sin_signed.new_zeros((T, self.nkv, self.hd))), dim=1)
         g = self.nh // self.nkv
         mask = self.mask.index_select(0, pos_idx).repeat(g, 1).unsqueeze(0).expand(self.nkv, g * T, self.max_len)
         for li in range(len(self.layers)):
@@ -146,8 +151,7 @@ class GraphDecoder:
             raise ValueError(f"prompt length {T} outside 1..{self.max_len - 1}")
         self.stream.wait_stream(torch.cuda.current_stream(self.dev))     # the ids may still be in flight there
         with torch.cuda.stream(self.stream):
-            self.kcache.zero_()
-            self.vcache.zero_()
+            self.kvcache.zero_()
             pos_idx = torch.arange(T, device=self.dev)
             logits = self._forward(ids, pos_idx, precision)
             self.logits.copy_(logits)
@@ -164,7 +168,7 @@ class GraphDecoder:
         """Records the decode step for ``precision`` (state is saved and restored around the warm-up)."""
         if precision in self.graphs:
             return self.graphs[precision]
-        saved = (self.tok.clone(), self.pos.clone(), self.emitted.clone(), self.kcache.clone(), self.vcache.clone())
+        saved = (self.tok.clone(), self.pos.clone(), self.emitted.clone(), self.kvcache.clone())
         with torch.cuda.stream(self.stream):
             self.pos.clamp_(max=self.max_len - 4)
             for _ in range(2):
@@ -174,7 +178,7 @@ class GraphDecoder:
             with torch.cuda.graph(g, stream=self.stream):
                 self._step(precision)
         self.stream.synchronize()
-        for dst, src in zip((self.tok, self.pos, self.emitted, self.kcache, self.vcache), saved):
+        for dst, src in zip((self.tok, self.pos, self.emitted, self.kvcache), saved):
             dst.copy_(src)
         torch.cuda.synchronize()
         self.graphs[precision] = g
