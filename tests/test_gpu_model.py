@@ -85,3 +85,42 @@ def test_graph_decoder_matches_eager_and_the_dense_model(pair):
         top2 = want.float().topk(2).values
         if (top2[0] - top2[1]).item() > 4e-2 * want.abs().max().item():
             assert int(with_graph[-1]) == int(want.argmax())
+
+
+def test_opt_layout_with_biased_linears():
+    """A second module layout (the reference's analyzer/architectures/opt.yaml: model.decoder.layers,
+    q/k/v/out_proj, fc1, fc2) whose linears carry biases (AnyPrecisionLinear.py:40-46,68-69), through
+    from_config -> save_quantized -> from_quantized, against the dense model of the same weights."""
+    import tempfile
+    from transformers import OPTConfig, OPTForCausalLM
+    from any_precision_amd import AnyPrecisionForCausalLM
+
+    def config():
+        cfg = OPTConfig(hidden_size=64, ffn_dim=160, num_hidden_layers=2, num_attention_heads=4, vocab_size=320,
+                        max_position_embeddings=64, word_embed_proj_dim=64, do_layer_norm_before=True)
+        cfg.anyprec = {"seed_precision": 3, "parent_precision": 8, "group_count": 1,
+                       "arch_config": {"model_name": "model.decoder", "layers_name": "layers",
+                                       "module_names": ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj",
+                                                        "self_attn.out_proj", "fc1", "fc2"]}}
+        return cfg
+
+    ap = AnyPrecisionForCausalLM.from_config(config(), seed=2, device="cuda")
+    assert len(ap.ap_linears) == 12 and all(m.bias is not None for m in ap.ap_linears)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    for m in ap.ap_linears:                     # non-trivial biases
+        m.bias.copy_(torch.randn(m.bias.shape, device="cuda", generator=gen) * 0.05)
+    with tempfile.TemporaryDirectory() as d:
+        ap.save_quantized(d)
+        back = AnyPrecisionForCausalLM.from_quantized(d).cuda()
+    ids = torch.randint(0, 320, (1, 7), generator=torch.Generator().manual_seed(0)).cuda()
+    for b in (3, 8):
+        dense = OPTForCausalLM(config()).half().cuda().eval()
+        missing, unexpected = dense.load_state_dict(ap.dense_state_dict(b), strict=False)
+        assert not unexpected and not missing, (missing, unexpected)
+        with torch.inference_mode():
+            want = dense(ids).logits
+            got = ap(ids, precision=b).logits
+            got_back = back(ids, precision=b).logits
+        _close(got, want, f"opt b={b}")
+        assert torch.equal(got, got_back), "model reloaded from its checkpoint differs"
