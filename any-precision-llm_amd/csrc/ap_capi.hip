@@ -167,6 +167,8 @@ namespace {
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
 int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
              int w_bits, hipStream_t st) {
+    // the kernel addresses the activations with 32-bit byte offsets
+    if ((long long)M * K * 2 > 0xffffffffLL) return AP_ELIMIT;
     GemmGeometry geo;
     geo.mb = (M + 15) / 16;
     geo.grid = (N + 15) / 16;

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 
     // this wave's range of steps (4 * WPS words of every row per step)
     const int steps = (W + 4 * WPS - 1) / (4 * WPS);
-    const int s_begin = steps * ks / KS, s_end = steps * (ks + 1) / KS;  // steps <= 512
+    const int s_begin = steps * ks / KS, s_end = steps * (ks + 1) / KS;  // steps < 2^26, KS <= 8: no overflow
 
     const uint32_t *wrow = qweight + (size_t)row * W;
     // q[p][i]: plane p, i-th word of this lane for the step
