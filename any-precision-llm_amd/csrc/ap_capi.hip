@@ -24,6 +24,7 @@ struct Tuning {
     int force_gemm_split;   // > 0: K-split waves per workgroup of the fused GEMM
     int mfma4_mode;         // 4x4x4 matrix-core kernel: 0 never, 1 where it pays, 2 for 2..8 rows wherever it fits
     int force_gemv4_groups; // > 0: word groups per wave of that kernel
+    int gemm_rb2_mode;      // fused GEMM, two weight-row blocks per workgroup: 0 never, 1 where it pays, 2 always
 };
 
 int env_int(const char *name, int dflt) {
@@ -41,6 +42,7 @@ const Tuning &tuning() {
         env_int("AP_GEMM_SPLIT", 0),
         env_int("AP_MATMUL_MFMA4", 1),
         env_int("AP_GEMV4_GROUPS", 0),
+        env_int("AP_GEMM_RB2", 1),
     };
     return t;
 }
@@ -171,8 +173,18 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     if ((long long)M * K * 2 > 0xffffffffLL) return AP_ELIMIT;
     GemmGeometry geo;
     geo.mb = (M + 15) / 16;
-    geo.grid = (N + 15) / 16;
     const int W = K >> 5;
+    // Two blocks of 16 weight rows per workgroup halve the L2 traffic of the activations, which
+    // bounds this kernel, but also the number of workgroups, and they need twice the plane
+    // registers: measured faster from 9 activation rows on, on linears of at least 8192 rows -- at
+    // 3 bits, and at up to 5 bits (6 with two activation row blocks) when the linear has at least
+    // 56 M weights (14336 x 4096, 8192 x 8192, 28672 x 8192: 5-25 %).
+    const int rb_mode = tuning().gemm_rb2_mode;  // 0 never, 1 where it pays, 2 wherever the kernel allows
+    const bool rb_fits = (W & 3) == 0 && geo.mb <= 2 && N >= 32;
+    const bool rb_pays = M > 8 && N >= 8192 &&
+                         (w_bits == 3 || (w_bits <= (geo.mb == 2 ? 6 : 5) && (long long)N * K >= 56LL << 20));
+    geo.rb = (rb_fits && (rb_mode >= 2 || (rb_mode == 1 && rb_pays))) ? 2 : 1;
+    geo.grid = (N + 16 * geo.rb - 1) / (16 * geo.rb);
     const int steps = (W & 3) == 0 ? (W + 15) / 16 : (W + 3) / 4;  // the kernel's steps along K
     // As many K-split waves as a workgroup holds: every split measured slower with fewer
     // (the grid alone, N/16 workgroups, is far too small to fill 256 CUs).

@@ -55,18 +55,25 @@ __device__ __forceinline__ void transpose_rows4(uint32_t (&r)[4]) {
     r[3] = d[1];
 }
 
-// MB = activation row blocks of 16 (M <= 16*MB).  Grid: ceil(N/16) workgroups of (64, KS).
-template <int BITS, int MB, bool VEC4, int MP>
+// MB = activation row blocks of 16 (M <= 16*MB).  RB = blocks of 16 weight rows a wave works on in
+// lockstep: every activation operand it loads then feeds RB matrix instructions instead of one,
+// which divides the L2 traffic of the activations by RB -- at the price of 1/RB as many
+// workgroups, so only linears with many rows use RB = 2.  Grid: ceil(N / (16 RB)) workgroups of (64, KS).
+template <int BITS, int MB, bool VEC4, int MP, int RB>
 __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K) {
     constexpr int NC = 1 << BITS;
     constexpr int WPS = VEC4 ? 4 : 1;             // words per lane and step
-    constexpr int TQ = kGemmRows * NC / 8;  // 16-byte quads of the 16 tables
-    __shared__ __attribute__((aligned(16))) half_t tables[kGemmRows][NC];
-    __shared__ float red[kGemmMaxSplit][MB][4][kWave];
-    // activation staging, one private region per wave: MP rows x 16 octets (4 byte groups x 4 words)
-    __shared__ u32x4 xs[kGemmMaxSplit][MP > 0 ? MP * 16 : 1];
+    constexpr int ROWS = kGemmRows * RB;    // weight rows per workgroup
+    constexpr int TQ = ROWS * NC / 8;       // 16-byte quads of their tables
+    __shared__ __attribute__((aligned(16))) half_t tables[ROWS][NC];
+    // One private region per wave.  While the wave computes it stages activations there: MP rows x 16
+    // octets (4 byte groups x 4 words).  Afterwards the same bytes carry the wave's partial tiles
+    // (RB x MB x 4 x 64 floats) to the combine step -- LDS operations of one wave complete in order, so
+    // the wave's last operand reads are done before its tile is written.
+    constexpr int XS = MP * 16 > RB * MB * 64 ? MP * 16 : RB * MB * 64;
+    __shared__ u32x4 xs[kGemmMaxSplit][XS];
     static_assert(MP == 0 || (MP >= 8 && MP <= 16 * MB && (MP & (MP - 1)) == 0), "");
 
     const int lane = threadIdx.x;
@@ -74,39 +81,45 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const int col = lane & 15, grp = lane >> 4;
     const int W = K >> 5;
     const size_t plane_stride = (size_t)N * W;
-    const int n0 = blockIdx.x * kGemmRows;
-    const int row = min(n0 + col, N - 1);  // rows past N repeat row N-1 and are not stored
+    const int n0 = blockIdx.x * ROWS;
 
     // this wave's range of steps (4 * WPS words of every row per step)
     const int steps = (W + 4 * WPS - 1) / (4 * WPS);
     const int s_begin = steps * ks / KS, s_end = steps * (ks + 1) / KS;  // steps < 2^26, KS <= 8: no overflow
 
-    const uint32_t *wrow = qweight + (size_t)row * W;
-    // q[p][i]: plane p, i-th word of this lane for the step
-    auto fetch = [&](int step, uint32_t(&q)[BITS][WPS]) {
+    const uint32_t *wrow[RB];  // rows past N repeat row N-1 and are not stored
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) wrow[rb] = qweight + (size_t)min(n0 + rb * kGemmRows + col, N - 1) * W;
+    // q[rb][p][i]: row block rb, plane p, i-th word of this lane for the step
+    auto fetch = [&](int step, uint32_t(&q)[RB][BITS][WPS]) {
         if constexpr (VEC4) {
             // W % 4 == 0: a quad is entirely inside the row or entirely past its end (then it is
             // clamped to the last quad and never used)
             const int w = min(16 * step + 4 * grp, W - 4);
 #pragma unroll
-            for (int p = 0; p < BITS; p++) {
-                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow + p * plane_stride + w));
+            for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-                for (int i = 0; i < 4; i++) q[p][i] = v[i];
-            }
+                for (int p = 0; p < BITS; p++) {
+                    const u32x4 v =
+                        __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[rb] + p * plane_stride + w));
+#pragma unroll
+                    for (int i = 0; i < 4; i++) q[rb][p][i] = v[i];
+                }
         } else {
             // plain (temporal) loads: the 64-byte line is needed again by the next three steps
             const int w = min(4 * step + grp, W - 1);
 #pragma unroll
-            for (int p = 0; p < BITS; p++) q[p][0] = wrow[p * plane_stride + w];
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int p = 0; p < BITS; p++) q[rb][p][0] = wrow[rb][p * plane_stride + w];
         }
     };
 
     // Load order: planes of the first step, then the tables -- both are in flight together
-    // and the tables are staged while nothing else could run anyway.  The 16 tables are
-    // contiguous in lut (rows past N re-read the last 16 bytes of the array; their columns
-    // are never stored).
-    uint32_t qn[BITS][WPS];
+    // and the tables are staged while nothing else could run anyway.  The tables of the
+    // workgroup's rows are contiguous in lut (rows past N re-read the last 16 bytes of the
+    // array; their columns are never stored).
+    uint32_t qn[RB][BITS][WPS];
     if (s_begin < s_end) fetch(s_begin, qn);
     {
         const int nthr = KS * kWave;
@@ -118,7 +131,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     __syncthreads();
     // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
     typedef __attribute__((address_space(3))) half_t lds_half_t;
-    const uint32_t tab_base = (uint32_t)(uintptr_t)((lds_half_t *)&tables[0][0]) + (uint32_t)col * (NC * 2);
+    const uint32_t tab_base0 = (uint32_t)(uintptr_t)((lds_half_t *)&tables[0][0]) + (uint32_t)col * (NC * 2);
 
     // byte offset of this lane's activation row in each row block (rows past M repeat row M-1)
     uint32_t xoff[MB];
@@ -127,9 +140,11 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const int full_chunks = W >> 5;                // chunks of 32 words; a shorter one may follow
     const uint32_t tail_stride = (uint32_t)(W & 31) * 16u;  // bytes of x between byte groups in the tail chunk
 
-    float4_t acc[MB];
+    float4_t acc[RB][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) acc[mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++) acc[rb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     // One step: transpose the planes of each word to indices, gather, multiply.  CHECK: the
     // step may reach past the end of the row (only the last step of a row can).
@@ -147,7 +162,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     constexpr int OCT = 4 * WPS;
     constexpr int AHEAD = MB == 1 ? 4 : (MB == 2 ? 2 : 1);
     constexpr int NL = MP / 4;  // staging loads per lane and word group
-    auto process = [&](auto check_c, int step, uint32_t(&q)[BITS][WPS]) {
+    auto process = [&](auto check_c, int step, uint32_t(&q)[RB][BITS][WPS]) {
         constexpr bool CHECK = decltype(check_c)::value;
         // x byte offset of byte group 0 of each word, and the distance between byte groups
         uint32_t kb[WPS], jstride[WPS];
@@ -203,11 +218,13 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
         static_for<AHEAD>([&](auto t_c) { load_a(t_c); });
         if constexpr (VEC4) {
 #pragma unroll
-            for (int p = 0; p < BITS; p++) transpose_rows4(q[p]);
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int p = 0; p < BITS; p++) transpose_rows4(q[rb][p]);
         }
         // index bytes hold the byte offset into the table (index * 2) where that fits a byte
         constexpr int PRE = BITS <= 7 ? 1 : 0;
-        uint32_t idx[8];
+        uint32_t idx[RB][8];
         static_for<OCT>([&](auto t_c) {
             constexpr int t = decltype(t_c)::value, wi = t / 4, j = t % 4, c = 3 - j;
             load_a(std::integral_constant<int, t + AHEAD>{});
@@ -216,30 +233,38 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
                     stage_store();
                     if constexpr (wi + 1 < WPS) stage_load(wi + 1);
                 }
-                uint32_t qq[BITS];
 #pragma unroll
-                for (int p = 0; p < BITS; p++) qq[p] = q[p][wi];
-                planes_to_indices<BITS, PRE>(qq, idx);
-            }
-            // B operand: the eight weights of byte group j
-            u32x4 bw;
-            static_for<4>([&](auto e_c) {
-                constexpr int i = decltype(e_c)::value;
-                uint32_t a0, a1;
-                if constexpr (PRE) {
-                    a0 = byte_add<c>(tab_base, idx[2 * i]);
-                    a1 = byte_add<c>(tab_base, idx[2 * i + 1]);
-                } else {
-                    a0 = tab_base + byte_offset<c, 1>(idx[2 * i]);
-                    a1 = tab_base + byte_offset<c, 1>(idx[2 * i + 1]);
+                for (int rb = 0; rb < RB; rb++) {
+                    uint32_t qq[BITS];
+#pragma unroll
+                    for (int p = 0; p < BITS; p++) qq[p] = q[rb][p][wi];
+                    planes_to_indices<BITS, PRE>(qq, idx[rb]);
                 }
-                half2_t h;
-                h.x = *reinterpret_cast<const lds_half_t *>(a0);
-                h.y = *reinterpret_cast<const lds_half_t *>(a1);
-                const uint32_t packed = __builtin_bit_cast(uint32_t, h);
-                bw[i] = live[wi] ? packed : 0u;
+            }
+            // B operands: the eight weights of byte group j of each row block
+            half8_t bfrag[RB];
+            static_for<RB>([&](auto rb_c) {
+                constexpr int rb = decltype(rb_c)::value;
+                const uint32_t tab_base = tab_base0 + rb * (kGemmRows * NC * 2);
+                u32x4 bw;
+                static_for<4>([&](auto e_c) {
+                    constexpr int i = decltype(e_c)::value;
+                    uint32_t a0, a1;
+                    if constexpr (PRE) {
+                        a0 = byte_add<c>(tab_base, idx[rb][2 * i]);
+                        a1 = byte_add<c>(tab_base, idx[rb][2 * i + 1]);
+                    } else {
+                        a0 = tab_base + byte_offset<c, 1>(idx[rb][2 * i]);
+                        a1 = tab_base + byte_offset<c, 1>(idx[rb][2 * i + 1]);
+                    }
+                    half2_t h;
+                    h.x = *reinterpret_cast<const lds_half_t *>(a0);
+                    h.y = *reinterpret_cast<const lds_half_t *>(a1);
+                    const uint32_t packed = __builtin_bit_cast(uint32_t, h);
+                    bw[i] = live[wi] ? packed : 0u;
+                });
+                bfrag[rb] = __builtin_bit_cast(half8_t, bw);
             });
-            const half8_t bfrag = __builtin_bit_cast(half8_t, bw);
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) {
                 half8_t afrag;
@@ -250,21 +275,25 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
                 } else {
                     afrag = a[t][mb];
                 }
-                acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag, acc[mb], 0, 0, 0);
+#pragma unroll
+                for (int rb = 0; rb < RB; rb++)
+                    acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag[rb], acc[rb][mb], 0, 0, 0);
             }
         });
     };
 
     // With few planes the next step's words are fetched while this step computes; with
     // many, the second register set is not worth its registers (no measurable gain).
-    constexpr bool PREFETCH = BITS * WPS <= 20;
+    constexpr bool PREFETCH = RB * BITS * WPS <= 20;
     for (int step = s_begin; step < s_end; step++) {
-        uint32_t q[BITS][WPS];
+        uint32_t q[RB][BITS][WPS];
         if (PREFETCH || step == s_begin) {
 #pragma unroll
-            for (int p = 0; p < BITS; p++)
+            for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-                for (int i = 0; i < WPS; i++) q[p][i] = qn[p][i];
+                for (int p = 0; p < BITS; p++)
+#pragma unroll
+                    for (int i = 0; i < WPS; i++) q[rb][p][i] = qn[rb][p][i];
         } else {
             fetch(step, q);
         }
@@ -277,17 +306,20 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 
     // Combine the K-split partial tiles in wave order (also with one wave: it keeps the
     // accumulator indices static).  D[i][j]: lane l holds rows i = 4 (l / 16) + v, column l % 16.
+    float *mine = reinterpret_cast<float *>(&xs[ks][0]);
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+    for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) red[ks][mb][v][lane] = acc[mb][v];
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) mine[((rb * MB + mb) * 4 + v) * kWave + lane] = acc[rb][mb][v];
     __syncthreads();
-    for (int t = ks; t < MB * 4; t += KS) {
-        const int mb = t >> 2, v = t & 3;
+    for (int t = ks; t < RB * MB * 4; t += KS) {
+        const int rb = t / (MB * 4), mb = (t >> 2) % MB, v = t & 3;
         float sum = 0.f;
-        for (int kk = 0; kk < KS; kk++) sum += red[kk][mb][v][lane];
-        const int m = mb * 16 + 4 * grp + v;
-        if (m < M && n0 + col < N) out[(size_t)m * N + n0 + col] = (half_t)sum;
+        for (int kk = 0; kk < KS; kk++) sum += reinterpret_cast<const float *>(&xs[kk][0])[t * kWave + lane];
+        const int m = mb * 16 + 4 * grp + v, n = n0 + rb * kGemmRows + col;
+        if (m < M && n < N) out[(size_t)m * N + n] = (half_t)sum;
     }
 }
 

@@ -19,13 +19,18 @@ void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qwe
     // 10-17 % faster at every bit-width); one row block is as fast or faster straight from
     // global memory, and beyond two the staging region would crowd out the second workgroup
     // of a CU.
-#define AP_GEMM_LAUNCH(MBV, MPV)                                                                                  \
-    do {                                                                                                          \
-        if (vec4) gemm_kbit_kernel<BITS, MBV, true, MPV><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);   \
-        else gemm_kbit_kernel<BITS, MBV, false, MPV><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);       \
+#define AP_GEMM_LAUNCH(MBV, MPV)                                                                                     \
+    do {                                                                                                             \
+        if (vec4) gemm_kbit_kernel<BITS, MBV, true, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);   \
+        else gemm_kbit_kernel<BITS, MBV, false, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);       \
     } while (0)
 #define AP_GEMM_CASE(MBV) \
     case MBV: AP_GEMM_LAUNCH(MBV, 0); break;
+    if (geo.rb == 2) {  // chosen by the caller only with vec4 and at most two activation row blocks
+        if (geo.mb == 1) gemm_kbit_kernel<BITS, 1, true, 0, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+        else gemm_kbit_kernel<BITS, 2, true, 32, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+        return;
+    }
     switch (geo.mb) {
         AP_GEMM_CASE(1)
         case 2: AP_GEMM_LAUNCH(2, 32); break;

@@ -12,10 +12,11 @@ constexpr int kGemmMaxSplit = 8;  // K-split waves per workgroup
 struct GemmGeometry {
     int mb;    // activation row blocks of 16
     int ks;    // K-split waves per workgroup
-    int grid;  // workgroups (16 weight rows each)
+    int rb;    // blocks of 16 weight rows per workgroup: 1, or 2 (only with K % 128 == 0 and mb <= 2)
+    int grid;  // workgroups = ceil(N / (16 rb))
 };
 
-// Launches gemm_kbit_kernel<BITS, geo.mb> on `stream`.
+// Launches gemm_kbit_kernel<BITS, geo.mb, ..., geo.rb> on `stream`.
 template <int BITS>
 void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int M, int N, int K, hipStream_t stream);
