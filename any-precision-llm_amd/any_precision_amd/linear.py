@@ -5,8 +5,8 @@ Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]
 ``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
 ``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
 Batch dispatch: up to 8 activation rows -> ``matmul_kbit`` as in the reference (:60-64);
-9 .. ``FUSED_GEMM_ROWS`` rows -> the fused ``gemm_kbit``; beyond -> ``dequant_kbit`` +
-``torch.matmul`` as in the reference.
+9 .. 32 rows (.. 64 where ``fused_gemm_pays`` says so) -> the fused ``gemm_kbit``; beyond ->
+``dequant_kbit`` + ``torch.matmul`` as in the reference.
 """
 from __future__ import annotations
 
@@ -19,10 +19,14 @@ except ModuleNotFoundError:
     matmul_kbit, matmul_kbit_group, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, None, 0
 
 
-# Up to this many activation rows the fused GEMM beats dequant_kbit + torch.matmul on every
-# Llama-2-7B shape and bit-width measured (1.3-2.6x at 16 rows); beyond, the re-read of the
-# activations per 16 weight rows costs more than materialising the weight once.
-FUSED_GEMM_ROWS = min(32, GEMM_MAX_M)
+def fused_gemm_pays(rows: int, out_features: int, w_bits: int) -> bool:
+    """Whether the fused GEMM beats dequant_kbit + torch.matmul (measured on the Llama-2-7B / Llama-3-8B
+    / 8192 x 8192 shapes, every bit-width): always up to 32 activation rows (1.3-2.6x at 16); up to 64
+    on linears of fewer than 8192 rows, and on larger ones at up to 5 bits.  Beyond, the re-read of
+    the activations per block of weight rows costs more than materialising the weight once."""
+    if rows <= min(32, GEMM_MAX_M):
+        return True
+    return rows <= min(64, GEMM_MAX_M) and (out_features < 8192 or w_bits <= 5)
 
 
 def forward_group(modules, x, precision=None, concat=False):
@@ -92,7 +96,7 @@ class AnyPrecisionLinear(nn.Module):
         rows = x.numel() // x.shape[-1]
         if rows <= 8:
             x = matmul_kbit(x, self.qweight, lut, w_bits)
-        elif rows <= FUSED_GEMM_ROWS and x.is_contiguous():
+        elif fused_gemm_pays(rows, self.out_features, w_bits) and x.is_contiguous():
             x = gemm_kbit(x, self.qweight, lut, w_bits)      # fused dequant -> MFMA, weight never materialised
         else:
             weight = dequant_kbit(self.qweight, lut, w_bits)

@@ -180,10 +180,20 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     // 3 bits, and at up to 5 bits (6 with two activation row blocks) when the linear has at least
     // 56 M weights (14336 x 4096, 8192 x 8192, 28672 x 8192: 5-25 %).
     const int rb_mode = tuning().gemm_rb2_mode;  // 0 never, 1 where it pays, 2 wherever the kernel allows
-    const bool rb_fits = (W & 3) == 0 && geo.mb <= 2 && N >= 32;
+    const bool rb_fits = (W & 3) == 0 && N >= 32;
     const bool rb_pays = M > 8 && N >= 8192 &&
-                         (w_bits == 3 || (w_bits <= (geo.mb == 2 ? 6 : 5) && (long long)N * K >= 56LL << 20));
+                         (w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (long long)N * K >= 56LL << 20));
     geo.rb = (rb_fits && (rb_mode >= 2 || (rb_mode == 1 && rb_pays))) ? 2 : 1;
+    if (geo.rb == 2 && geo.mb > 2) {
+        // the two-block variant exists for up to 32 activation rows: more go in chunks of 32 (the
+        // planes are re-read per chunk, which still costs less than one launch of the one-block variant)
+        for (int m0 = 0; m0 < M; m0 += 32) {
+            const int r = run_gemm(x + (size_t)m0 * K, qweight, lut, out + (size_t)m0 * N, M - m0 < 32 ? M - m0 : 32, N, K,
+                                   w_bits, st);
+            if (r != AP_OK) return r;
+        }
+        return AP_OK;
+    }
     geo.grid = (N + 16 * geo.rb - 1) / (16 * geo.rb);
     const int steps = (W & 3) == 0 ? (W + 15) / 16 : (W + 3) / 4;  // the kernel's steps along K
     // As many K-split waves as a workgroup holds: every split measured slower with fewer

@@ -129,7 +129,7 @@ def test_two_weight_row_blocks_per_workgroup_give_the_same_bits(ext, oracle, tmp
     """Large linears run the MFMA kernel with two blocks of 16 weight rows per workgroup; AP_GEMM_RB2=2
     (read once per process) forces that variant on the small ragged shapes a test can check against
     the oracle.  Each output is still summed in the same order, so the results must equal the
-    one-block variant's bit for bit."""
+    one-block variant's bit for bit.  More than 32 activation rows go through it in chunks of 32."""
     import os
     import subprocess
     import sys
@@ -145,7 +145,7 @@ for N, K in %r:
     L = make(N, K, seed=N + K)
     q, luts = layer_to_gpu(L)
     for b in range(3, 9):
-        for M in (9, 16, 20, 32):
+        for M in (9, 16, 20, 32, 40, 100):
             print(f"two row blocks N={N} K={K} b={b} M={M}", flush=True)
             x = synth.make_x(M, K, seed=M)
             got = ext.gemm_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
@@ -166,6 +166,6 @@ print("ok")
         L = make(N, K, seed=N + K)
         q, luts = layer_to_gpu(L)
         for b in range(3, 9):
-            for M in (9, 16, 20, 32):
+            for M in (9, 16, 20, 32, 40, 100):
                 _, xg = _x(M, K, seed=M)
                 assert torch.equal(ext.gemm_kbit(xg, q, luts[b], b).cpu(), forced[f"{N}_{K}_{b}_{M}"]), (N, K, b, M)
