@@ -67,10 +67,11 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     const Tuning &t = tuning();
     const int W = K >> 5;
     // One word per lane (two waves per 4096 elements of a row) measured 5-15 % faster than
-    // two on planes that come from HBM; two words per lane only when one would need more
-    // waves than a workgroup holds.
+    // two on planes that come from HBM, up to rows of 16384 elements; beyond (more than 8 waves
+    // per row) two words per lane are 7-10 % faster (8192 x 28672), and they are needed when
+    // one word per lane would take more waves than a workgroup holds.
     int wpl = 1;
-    if (M <= 2 && (W & 1) == 0 && (W + kWave - 1) / kWave > kGemvMaxSeg) wpl = 2;
+    if (M <= 2 && (W & 1) == 0 && (W + kWave - 1) / kWave > 8) wpl = 2;
     if (t.force_wpl == 1 || (t.force_wpl == 2 && (W & 1) == 0 && M <= 2)) wpl = t.force_wpl;
     const int seg = kWave * wpl;
     const int S = (W + seg - 1) / seg;
