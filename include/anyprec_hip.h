@@ -67,7 +67,8 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
 /* Fused dequant -> MFMA GEMM, 1 <= M <= 128: out[M,N] = x[M,K] . dequant(qweight, lut)^T
  * without materialising the fp16 weight.  No single counterpart in the reference: it is the
  * M > 8 branch of AnyPrecisionLinear.forward (AnyPrecisionLinear.py:60-62: dequant_kbit,
- * main.cu:60-91, then torch.matmul) in one launch.  fp32 accumulation, fp16 result. */
+ * main.cu:60-91, then torch.matmul) fused (one launch; more than 32 rows may run as launches
+ * of 32 rows each, in order, on the same stream).  fp32 accumulation, fp16 result. */
 int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int M, int N, int K, int w_bits, void *stream);
 
