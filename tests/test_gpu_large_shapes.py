@@ -48,9 +48,10 @@ def test_llama70b_mlp_shapes(N, K):
         del want_w
 
 
-def test_llama3_8b_mlp_shape_at_every_batch_up_to_eight():
+def test_llama3_8b_mlp_shape_under_the_default_routing():
     """14336 x 4096 at M = 1..8 under the default routing: the dot-product kernel (1, 2 and part of
-    3), the 4x4x4 matrix-core kernel with one (3, 4) and two (5..8) groups of activation rows."""
+    3), the 4x4x4 matrix-core kernel with one (3, 4) and two (5..8) groups of activation rows; then the
+    fused GEMM at 16, 32 and 48 rows."""
     import any_precision_ext as ext
     N, K = 14336, 4096
     gen = torch.Generator(device="cuda")
@@ -66,4 +67,13 @@ def test_llama3_8b_mlp_shape_at_every_batch_up_to_eight():
             got = ext.matmul_kbit(x, q, lut, b).double()
             assert (got - want).norm() <= REL_TOL * want.norm(), f"M={M} b={b}"
             assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"M={M} b={b}"
+        # the fused GEMM under its default routing: two weight-row blocks per workgroup at up to 5 / 6
+        # bits, chunks of 32 activation rows above 32
+        for M in (16, 32, 48):
+            print(f"llama3 mlp gemm b={b} M={M}", flush=True)
+            x = torch.randn((M, K), device="cuda", generator=gen).half()
+            want = x.double() @ want_w.T
+            got = ext.gemm_kbit(x, q, lut, b).double()
+            assert (got - want).norm() <= REL_TOL * want.norm(), f"gemm M={M} b={b}"
+            assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"gemm M={M} b={b}"
         del want_w
