@@ -373,6 +373,12 @@ def main():
             "sample": "torch CPU ops, 4096x4096, w_bits 3 and 8, batch 1: unpack + gather + matmul once; matmul "
                       "alone on the dequantised fp32 weight, mean of 5"}
 
+    if machine:
+        # how much of a step is the fixed cost of its 42 dependent launches, and the rate of the rest
+        floor_ms = len(BITS) * len(shapes) * machine["graph_node_us"] / 1e3
+        machine["step_launch_floor_ms"] = round(floor_ms, 4)
+        if ms_per_step > floor_ms:
+            machine["GBps_beyond_launch_floor"] = round(step_bytes / (ms_per_step - floor_ms) / 1e6, 1)
     result = {
         "metric": "bitplane GEMV effective HBM GB/s, Llama-2-7B layer set, w_bits 3-8, batch 1",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
