@@ -46,3 +46,13 @@ def test_cpu_tensors_are_rejected_not_computed():
         ext.dequant_kbit(q, l, 3)
     with pytest.raises(ValueError, match="GPU"):
         ext.matmul_kbit(torch.zeros(1, 64, dtype=torch.float16), q, l, 3)
+
+
+def test_fused_gemm_dispatch_rule():
+    """AnyPrecisionLinear sends 9..32 rows to the fused GEMM always, 33..64 only to small linears or
+    at up to 5 bits, more never (the reference sends everything above 8 rows to dequant + matmul,
+    AnyPrecisionLinear.py:60-62)."""
+    from any_precision_amd.linear import fused_gemm_pays
+    assert all(fused_gemm_pays(m, n, b) for m in (9, 32) for n in (4096, 14336) for b in (3, 8))
+    assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6)
+    assert not fused_gemm_pays(65, 4096, 3)

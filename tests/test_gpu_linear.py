@@ -31,12 +31,12 @@ def test_state_dict_keys_shapes_dtypes():
     assert m.precision == 8 and m.precisions == list(range(3, 9))
 
 
-def test_forward_both_branches_and_bias(oracle):
+def test_forward_every_branch_and_bias(oracle):
     L = make(128, 4096, seed=1)
     m, sd = _module(L)
     bias = sd["bias"].numpy().astype(np.float64)
     for b in (3, 5, 8):
-        for M in (1, 8, 9, 32, 33, 130):
+        for M in (1, 8, 9, 32, 33, 64, 65, 130):      # GEMV | fused GEMM (to 64 rows here) | dequant + matmul
             x = synth.make_x(M, L.K, seed=M)
             y = m(torch.from_numpy(x).cuda(), precision=b)
             _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
