@@ -53,57 +53,64 @@ def forward_group(modules, x, precision=None, concat=False):
 
 
 class AnyPrecisionLinear(nn.Module):
+    """One bitplane-packed linear layer serving every precision in ``precisions``.
+
+    Interface of the reference module (AnyPrecisionLinear.py:10-78): constructor arguments, the
+    ``qweight`` / ``lut{b}`` / ``bias`` buffers and hence the state-dict keys, ``forward(x,
+    precision=b)``, ``set_precision``, ``prune_precisions``, and the messages of its errors."""
+
     def __init__(self, in_features, out_features, supported_bits, bias=True, precisions=None, device=None,
                  dtype=None):
         super().__init__()
-        if dequant_kbit is None or matmul_kbit is None:
+        if matmul_kbit is None or dequant_kbit is None:
             raise ModuleNotFoundError("libanyprec_hip.so is not built: run `python any-precision-llm_amd/build.py`.")
-        if precisions is None:
-            precisions = supported_bits
-        if not isinstance(precisions, list):
-            raise RuntimeError("supported_bits must be a list of integers.")
-        if dtype is not None and dtype != torch.float16:
-            raise RuntimeError("Only float16 is supported for now.")
-        if in_features % 32 != 0:
-            raise RuntimeError("in_features must be a multiple of 32.")
-
-        self.in_features = in_features
-        self.out_features = out_features
-        self.precisions = precisions
-        self.precision = max(self.precisions)
+        precisions = supported_bits if precisions is None else precisions
+        self._validate(in_features, precisions, dtype)
+        self.in_features, self.out_features = in_features, out_features
         self.supported_bits = supported_bits
-
-        self.register_buffer(
-            "qweight",
-            torch.empty((max(supported_bits), out_features, in_features // 32), dtype=torch.int32, device=device),
-        )
-        for bit in supported_bits:
-            self.register_buffer(f"lut{bit}", torch.empty((out_features, 2 ** bit), dtype=dtype, device=device))
+        self.precisions = precisions
+        self.precision = max(precisions)          # AnyPrecisionLinear.py:26: the widest by default
+        # plane p of the parent code is qweight[p] (plane 0 = most significant bit): [P, N, K/32] int32
+        planes = torch.empty((max(supported_bits), out_features, in_features // 32), dtype=torch.int32, device=device)
+        self.register_buffer("qweight", planes)
+        # one table of 2**b centroids per row and supported bit-width
+        for b in supported_bits:
+            self.register_buffer(f"lut{b}", torch.empty((out_features, 1 << b), dtype=dtype, device=device))
+        # a buffer, not a parameter, as in the reference (:40-46): it is loaded, never trained
         if bias:
             self.register_buffer("bias", torch.empty((out_features,), dtype=dtype, device=device))
         else:
             self.bias = None
 
+    @staticmethod
+    def _validate(in_features, precisions, dtype):
+        if not isinstance(precisions, list):
+            raise RuntimeError("supported_bits must be a list of integers.")
+        if dtype not in (None, torch.float16):
+            raise RuntimeError("Only float16 is supported for now.")
+        if in_features % 32:
+            raise RuntimeError("in_features must be a multiple of 32.")
+
     def prune_precisions(self):
+        """Drops what no precision in ``precisions`` reads: planes below the widest one kept and the
+        tables of the other bit-widths (AnyPrecisionLinear.py:48-52)."""
         self.qweight = self.qweight[:max(self.precisions)]
-        for bit in self.supported_bits:
-            if bit not in self.precisions:
-                delattr(self, f"lut{bit}")
+        for b in set(self.supported_bits) - set(self.precisions):
+            delattr(self, f"lut{b}")
 
     def forward(self, x, **kwargs):
-        w_bits = kwargs["precision"] if "precision" in kwargs else self.precision
-        lut = self._buffers[f"lut{w_bits}"]
+        w_bits = kwargs.get("precision", self.precision)
+        table = self._buffers[f"lut{w_bits}"]
         rows = x.numel() // x.shape[-1]
-        if rows <= 8:
-            x = matmul_kbit(x, self.qweight, lut, w_bits)
+        if rows <= 8:                                       # GEMV / skinny kernels (reference: :63-64)
+            y = matmul_kbit(x, self.qweight, table, w_bits)
         elif fused_gemm_pays(rows, self.out_features, w_bits) and x.is_contiguous():
-            x = gemm_kbit(x, self.qweight, lut, w_bits)      # fused dequant -> MFMA, weight never materialised
-        else:
-            weight = dequant_kbit(self.qweight, lut, w_bits)
-            x = torch.matmul(x, weight.T)
+            y = gemm_kbit(x, self.qweight, table, w_bits)   # fused dequant -> MFMA, weight never materialised
+        else:                                               # reference: :60-62
+            y = torch.matmul(x, dequant_kbit(self.qweight, table, w_bits).T)
         if self.bias is not None:
-            x += self.bias
-        return x
+            y += self.bias
+        return y
 
     def set_precision(self, precision):
         if precision not in self.precisions:
@@ -111,4 +118,5 @@ class AnyPrecisionLinear(nn.Module):
         self.precision = precision
 
     def extra_repr(self) -> str:
-        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}"
+        return (f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, "
+                f"precisions={self.precisions}")
