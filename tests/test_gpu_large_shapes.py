@@ -77,3 +77,23 @@ def test_llama3_8b_mlp_shape_under_the_default_routing():
             assert (got - want).norm() <= REL_TOL * want.norm(), f"gemm M={M} b={b}"
             assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"gemm M={M} b={b}"
         del want_w
+
+
+@pytest.mark.parametrize("N,K", [(2560, 2560), (10240, 2560), (2560, 10240)])
+def test_phi2_shapes_against_the_oracle(N, K, oracle):
+    """Linear shapes of Phi-2 (hidden 2560: rows of 2.5 chunks, tail chunk of 16 words; the reference's
+    analyzer/architectures/phi.yaml lists the model) through every op, against the oracle."""
+    import numpy as np
+    import any_precision_ext as ext
+    from _util import assert_bit_exact, assert_close_gemv, layer_to_gpu, make
+    from any_precision_amd import synth
+    L = make(N, K, seed=N // 10 + K)
+    q, luts = layer_to_gpu(L)
+    for b in (3, 5, 8):
+        print(f"phi2 N={N} K={K} b={b}", flush=True)
+        want_w = np.take_along_axis(L.luts[b], (L.codes >> (8 - b)).astype(np.int64), axis=1)
+        assert_bit_exact(ext.dequant_kbit(q, luts[b], b), want_w, f"dequant N={N} K={K} b={b}")
+        for M, fn in ((1, ext.matmul_kbit), (4, ext.matmul_kbit), (8, ext.matmul_kbit), (16, ext.gemm_kbit)):
+            x = synth.make_x(M, K, seed=M)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(fn(torch.from_numpy(x).cuda(), q, luts[b], b), want, f"{fn.__name__} N={N} K={K} b={b} M={M}")
