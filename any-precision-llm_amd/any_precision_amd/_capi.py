@@ -11,8 +11,8 @@ _PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libanyprec_hip.so")
 
 AP_OK = 0
-AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT = -1, -2, -3, -4, -5, -6
-AP_ABI_VERSION = 2
+AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT, AP_EKNOB = -1, -2, -3, -4, -5, -6, -7
+AP_ABI_VERSION = 3
 
 if not os.path.exists(LIB_PATH):
     raise ModuleNotFoundError(
@@ -39,6 +39,14 @@ lib.ap_matmul_kbit_group.argtypes = [_vp, _ci, _pvp, _pvp, _pvp, _pi, _ci, _ci, 
 lib.ap_matmul_kbit_group.restype = _ci
 lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi]
 lib.ap_matmul_kbit_geometry.restype = _ci
+lib.ap_probe_stream.argtypes = [_vp, ctypes.c_longlong, _vp, ctypes.c_longlong, _vp, _ci, _vp]
+lib.ap_probe_stream.restype = _ci
+lib.ap_probe_empty.argtypes = [_vp, _vp]
+lib.ap_probe_empty.restype = _ci
+lib.ap_set_tuning.argtypes = [ctypes.c_char_p, _ci]
+lib.ap_set_tuning.restype = _ci
+lib.ap_get_tuning.argtypes = [ctypes.c_char_p, _pi]
+lib.ap_get_tuning.restype = _ci
 
 if lib.ap_abi_version() != AP_ABI_VERSION:
     raise ImportError(
@@ -46,7 +54,7 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
     )
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
-           "ap_gemm_kbit", "ap_matmul_kbit_geometry")
+           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
 
@@ -76,3 +84,33 @@ def matmul_geometry(M: int, N: int, K: int, w_bits: int) -> dict:
     vals = [ctypes.c_int() for _ in range(4)]
     check(lib.ap_matmul_kbit_geometry(M, N, K, w_bits, *[ctypes.byref(v) for v in vals]), "ap_matmul_kbit_geometry")
     return dict(zip(("wpl", "segments", "rows", "grid"), (v.value for v in vals)))
+
+
+def set_tuning(name: str, value: int) -> None:
+    """ap_set_tuning: override one launch-heuristic knob for this process (tests, benchmarks)."""
+    check(lib.ap_set_tuning(name.encode(), int(value)), f"ap_set_tuning({name})")
+
+
+def get_tuning(name: str) -> int:
+    val = ctypes.c_int()
+    check(lib.ap_get_tuning(name.encode(), ctypes.byref(val)), f"ap_get_tuning({name})")
+    return val.value
+
+
+class tuning:
+    """Context manager: `with tuning(gemm_rb2=2): ...` sets knobs and restores them on exit."""
+
+    def __init__(self, **knobs):
+        self.knobs = knobs
+        self.saved = {}
+
+    def __enter__(self):
+        for k, v in self.knobs.items():
+            self.saved[k] = get_tuning(k)
+            set_tuning(k, v)
+        return self
+
+    def __exit__(self, *exc):
+        for k, v in self.saved.items():
+            set_tuning(k, v)
+        return False

@@ -155,4 +155,42 @@ AP_HD void planes_to_pair_indices(const uint32_t (&q)[BITS], uint32_t (&pidx)[4]
     }
 }
 
+// Adjacent-pair form for BITS = 3, 4: apair[i], i = 0..3; byte b of apair[i] addresses the table entry
+// of the element PAIR (2i, 2i+1) of byte group 3 - b -- two elements that also share a dword of the
+// fp16 activations, so the activations need no rearranging (the form above pairs e with e + 4).
+// The byte holds the two indices bit-interleaved: with A = index(2i), B = index(2i+1) and A_k the bit
+// of weight 2^k,
+//     BITS = 4:  byte = A3 B3 A2 B2 A1 B1 A0 B0                       (entry number of a 256-entry table)
+//     BITS = 3:  byte = A2 B2 A1 B1 A0 B0 0 0                         (BYTE OFFSET into 64 dword entries)
+// Built as a 4 x 4 transpose of the 2-bit blocks of every byte across the plane words: two butterfly
+// stages, 16 bit-ops for 4 planes and 14 for 3 (one row is zero).
+template <int BITS>
+AP_HD void planes_to_adjacent_pairs(const uint32_t (&q)[BITS], uint32_t (&apair)[4]) {
+    static_assert(BITS == 3 || BITS == 4, "pair tables exist for 3 and 4 bits");
+    // row k supplies block k of the output byte: the plane of weight 2^k (BITS = 4), or of weight 2^(k-1)
+    // with a zero row 0 (BITS = 3)
+    uint32_t r[4];
+    constexpr bool Z0 = BITS == 3;
+    r[0] = Z0 ? 0u : q[3];
+    r[1] = q[BITS - 1 - (Z0 ? 0 : 1)];
+    r[2] = q[BITS - 2 - (Z0 ? 0 : 1)];
+    r[3] = q[0];
+    swap_blocks<4, 0x0F0F0F0Fu, Z0, false>(r[0], r[2]);
+    swap_blocks<4, 0x0F0F0F0Fu>(r[1], r[3]);
+    swap_blocks<2, 0x33333333u>(r[0], r[1]);
+    swap_blocks<2, 0x33333333u>(r[2], r[3]);
+    // r[m] collects block m (bits 2m+1, 2m = elements 6-2m, 7-2m) of every plane: pair i = 3 - m
+#pragma unroll
+    for (int i = 0; i < 4; i++) apair[i] = r[3 - i];
+}
+
+// The two table indices a byte of planes_to_adjacent_pairs stands for (host and device; the kernels use
+// it to build their pair tables): first = index of element 2i, second = index of element 2i+1.
+template <int BITS>
+AP_HD void adjacent_pair_split(uint32_t byte, uint32_t &first, uint32_t &second) {
+    const uint32_t v = BITS == 3 ? byte >> 2 : byte;
+    first = ((v >> 1) & 1u) | ((v >> 2) & 2u) | ((v >> 3) & 4u) | ((v >> 4) & 8u);
+    second = (v & 1u) | ((v >> 1) & 2u) | ((v >> 2) & 4u) | ((v >> 3) & 8u);
+}
+
 }  // namespace ap

@@ -1,50 +1,66 @@
 // C ABI of libanyprec_hip: argument checks, launch geometry, dispatch.
 // The declarations and their reference counterparts are in include/anyprec_hip.h.
 #include <hip/hip_runtime.h>
-#include <stdlib.h>
+#include <string.h>
 
 #include "anyprec_hip.h"
 #include "ap_dequant.hpp"
 #include "ap_gemm_launch.hpp"
 #include "ap_gemv4_launch.hpp"
 #include "ap_gemv_launch.hpp"
+#include "ap_gemvf_launch.hpp"
+#include "ap_gemvp_launch.hpp"
+#include "ap_gemvr_launch.hpp"
+#include "ap_probe.hpp"
 
 namespace {
 
 using namespace ap;
 
-constexpr int kNumCUs = 256;  // MI355X: 8 XCDs x 32 CUs
-
-struct Tuning {
-    int target_waves;  // waves the GEMV grid aims for (rows per wave follows)
-    int force_rows;    // > 0: rows per wave, overrides target_waves
-    int force_wpl;     // > 0: words per lane
-    int dequant_blocks_per_cu;
-    int mfma_from_rows;     // ap_matmul_kbit uses the MFMA kernel from this many activation rows on
-    int force_gemm_split;   // > 0: K-split waves per workgroup of the fused GEMM
-    int mfma4_mode;         // 4x4x4 matrix-core kernel: 0 never, 1 where it pays, 2 for 2..8 rows wherever it fits
-    int force_gemv4_groups; // > 0: word groups per wave of that kernel
-    int gemm_rb2_mode;      // fused GEMM, two weight-row blocks per workgroup: 0 never, 1 where it pays, 2 always
+// Launch-heuristic knobs.  Defaults are what measured fastest on MI355X; ap_set_tuning() overrides one for
+// the whole process (tests force every kernel variant with it, benchmarks sweep with it).  Plain ints read
+// at every call: a caller that changes a knob while another thread launches gets either value.
+struct Knob {
+    const char *name;
+    int value;
 };
+enum {
+    kGemvTargetWaves,   // waves the dot-product GEMV grid aims for (rows per workgroup follows)
+    kGemvRows,          // > 0: rows per workgroup of that kernel, overrides the above
+    kGemvWpl,           // > 0: words per lane of that kernel
+    kDequantBlocksPerCu,
+    kMatmulMfmaFrom,    // ap_matmul_kbit uses the 16x16x32 MFMA kernel from this many activation rows on
+    kGemmSplit,         // > 0: K-split waves per workgroup of the fused GEMM
+    kMatmulMfma4,       // 4x4x4 matrix-core kernel: 0 never, 1 where it pays, 2 for 2..8 rows wherever it fits
+    kGemv4Groups,       // > 0: word groups per wave of that kernel
+    kGemmRb2,           // fused GEMM, two weight-row blocks per workgroup: 0 never, 1 where it pays, 2 always
+    kGemvStream,        // row-streaming GEMV: 0 never, 1 where it pays, 2 wherever it fits
+    kGemvStreamWaves,   // waves per CU the row-streaming GEMV grid aims for
+    kGemvFine,          // fine-grained row-pair GEMV: 0 never, 1 where it pays, 2 wherever it fits
+    kGemvPersist,       // persistent row-loop GEMV: 0 never, 1 where it pays, 2 wherever it fits
+    kGemvPersistWaves,  // waves per CU the persistent GEMV grid aims for
+    kKnobCount
+};
+Knob g_knobs[kKnobCount] = {
+    {"gemv_target_waves", 16384}, {"gemv_rows", 0},      {"gemv_wpl", 0},     {"dequant_blocks_per_cu", 32},
+    {"matmul_mfma_from", 5},      {"gemm_split", 0},     {"matmul_mfma4", 1}, {"gemv4_groups", 0},
+    {"gemm_rb2", 1},              {"gemv_stream", 1},    {"gemv_stream_waves", 24},
+    {"gemv_fine", 1},             {"gemv_persist", 1},   {"gemv_persist_waves", 8},
+};
+inline int knob(int k) { return __atomic_load_n(&g_knobs[k].value, __ATOMIC_RELAXED); }
 
-int env_int(const char *name, int dflt) {
-    const char *v = getenv(name);
-    return (v && *v) ? atoi(v) : dflt;
-}
-
-const Tuning &tuning() {
-    static const Tuning t = {
-        env_int("AP_GEMV_TARGET_WAVES", 16384),
-        env_int("AP_GEMV_ROWS", 0),
-        env_int("AP_GEMV_WPL", 0),
-        env_int("AP_DEQUANT_BLOCKS_PER_CU", 32),
-        env_int("AP_MATMUL_MFMA_FROM", 5),
-        env_int("AP_GEMM_SPLIT", 0),
-        env_int("AP_MATMUL_MFMA4", 1),
-        env_int("AP_GEMV4_GROUPS", 0),
-        env_int("AP_GEMM_RB2", 1),
-    };
-    return t;
+// Compute units of the current device (256 on MI355X), looked up once per device.
+int cu_count() {
+    constexpr int kMaxDev = 64;
+    static int cached[kMaxDev];  // 0 = not yet known
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return n;
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -64,7 +80,7 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
         rows += n[g];
     }
     if (M < 1 || M > 8) return AP_EBATCH;
-    const Tuning &t = tuning();
+    const int force_wpl = knob(kGemvWpl), force_rows = knob(kGemvRows), target_waves = knob(kGemvTargetWaves);
     const int W = K >> 5;
     // One word per lane (two waves per 4096 elements of a row) measured 5-15 % faster than
     // two on planes that come from HBM, up to rows of 16384 elements; beyond (more than 8 waves
@@ -72,14 +88,14 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // one word per lane would take more waves than a workgroup holds.
     int wpl = 1;
     if (M <= 2 && (W & 1) == 0 && (W + kWave - 1) / kWave > 8) wpl = 2;
-    if (t.force_wpl == 1 || (t.force_wpl == 2 && (W & 1) == 0 && M <= 2)) wpl = t.force_wpl;
+    if (force_wpl == 1 || (force_wpl == 2 && (W & 1) == 0 && M <= 2)) wpl = force_wpl;
     const int seg = kWave * wpl;
     const int S = (W + seg - 1) / seg;
     if (S > kGemvMaxSeg) return AP_ELIMIT;
     // One row per workgroup until that would launch more than target_waves waves, then two
     // (the second row reuses the activation registers; more rows lengthen the compute
     // tail).  From M = 3 on the activations are the larger load: always two rows.
-    int R = t.force_rows > 0 ? t.force_rows : (int)((rows * S + t.target_waves - 1) / t.target_waves);
+    int R = force_rows > 0 ? force_rows : (int)((rows * S + target_waves - 1) / (target_waves > 0 ? target_waves : 1));
     R = (R >= 2 || M > 2) ? 2 : 1;
     geo->wpl = wpl;
     geo->S = S;
@@ -102,11 +118,15 @@ template <int BITS>
 void launch_dequant(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream) {
     const int S = ((K >> 5) + kWave - 1) / kWave;  // 64-word segments per row
     long long blocks = ((long long)N * S + kDequantWaves - 1) / kDequantWaves;
-    const long long cap = (long long)kNumCUs * tuning().dequant_blocks_per_cu;
+    const long long cap = (long long)cu_count() * knob(kDequantBlocksPerCu);
     if (blocks > cap) blocks = cap;
     dequant_kbit_kernel<BITS><<<dim3((unsigned)blocks), dim3(kDequantWaves * kWave), 0, stream>>>(
         qweight, reinterpret_cast<const half_t *>(lut), reinterpret_cast<half_t *>(out), N, K);
 }
+
+// hipGetLastError() returns AND clears the thread's sticky error, whoever left it: an entry point
+// drains it before its first launch, so that launch_status() reports only what its own launches did.
+void drain_stale_error() { (void)hipGetLastError(); }
 
 int launch_status() {
     const hipError_t e = hipGetLastError();
@@ -128,10 +148,55 @@ const char *ap_strerror(int code) {
         case AP_EALIGN: return "pointer not 16-byte aligned";
         case AP_EBATCH: return "batch M outside the range this entry point serves";
         case AP_ELIMIT: return "size exceeds the launch geometry limits";
+        case AP_EKNOB: return "unknown tuning knob";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
     return "unknown error code";
+}
+
+int ap_set_tuning(const char *name, int value) {
+    if (!name) return AP_ENULL;
+    for (int k = 0; k < kKnobCount; k++)
+        if (strcmp(name, g_knobs[k].name) == 0) {
+            __atomic_store_n(&g_knobs[k].value, value, __ATOMIC_RELAXED);
+            return AP_OK;
+        }
+    return AP_EKNOB;
+}
+
+int ap_get_tuning(const char *name, int *value) {
+    if (!name || !value) return AP_ENULL;
+    for (int k = 0; k < kKnobCount; k++)
+        if (strcmp(name, g_knobs[k].name) == 0) {
+            *value = knob(k);
+            return AP_OK;
+        }
+    return AP_EKNOB;
+}
+
+int ap_probe_stream(const void *buf0, long long bytes0, const void *buf1, long long bytes1, uint32_t *sink,
+                    int waves_per_cu, void *stream) {
+    if (!buf0 || !sink || (bytes1 > 0 && !buf1)) return AP_ENULL;
+    if (bytes0 < 0 || bytes1 < 0 || (bytes0 & 15) || (bytes1 & 15)) return AP_ESHAPE;
+    if (!aligned16(buf0) || (bytes1 > 0 && !aligned16(buf1))) return AP_EALIGN;
+    if (waves_per_cu < 1) waves_per_cu = 8;
+    const long long units = (bytes0 + bytes1) >> 4;
+    long long blocks = (long long)cu_count() * waves_per_cu / kProbeWaves;
+    const long long need = (units + kProbeWaves * kWave - 1) / (kProbeWaves * kWave);
+    if (blocks > need) blocks = need;
+    if (blocks < 1) blocks = 1;
+    drain_stale_error();
+    probe_stream_kernel<<<dim3((unsigned)blocks), dim3(kProbeWaves * kWave), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const u32x4 *>(buf0), bytes0 >> 4, static_cast<const u32x4 *>(buf1), bytes1 >> 4, sink);
+    return launch_status();
+}
+
+int ap_probe_empty(uint32_t *sink, void *stream) {
+    if (!sink) return AP_ENULL;
+    drain_stale_error();
+    probe_empty_kernel<<<dim3(1), dim3(kWave), 0, static_cast<hipStream_t>(stream)>>>(sink);
+    return launch_status();
 }
 
 int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, int w_bits,
@@ -141,6 +206,7 @@ int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
     if (rc != AP_OK) return rc;
     if (!aligned16(qweight) || !aligned16(lut) || !aligned16(out)) return AP_EALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    drain_stale_error();
     switch (w_bits) {
         case 3: launch_dequant<3>(qweight, lut, out, N, K, st); break;
         case 4: launch_dequant<4>(qweight, lut, out, N, K, st); break;
@@ -180,7 +246,7 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     // registers: measured faster from 9 activation rows on, on linears of at least 8192 rows -- at
     // 3 bits, and at up to 5 bits (6 with two activation row blocks) when the linear has at least
     // 56 M weights (14336 x 4096, 8192 x 8192, 28672 x 8192: 5-25 %).
-    const int rb_mode = tuning().gemm_rb2_mode;  // 0 never, 1 where it pays, 2 wherever the kernel allows
+    const int rb_mode = knob(kGemmRb2);  // 0 never, 1 where it pays, 2 wherever the kernel allows
     const bool rb_fits = (W & 3) == 0 && N >= 32;
     const bool rb_pays = M > 8 && N >= 8192 &&
                          (w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (long long)N * K >= 56LL << 20));
@@ -199,7 +265,7 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     const int steps = (W & 3) == 0 ? (W + 15) / 16 : (W + 3) / 4;  // the kernel's steps along K
     // As many K-split waves as a workgroup holds: every split measured slower with fewer
     // (the grid alone, N/16 workgroups, is far too small to fill 256 CUs).
-    int ks = tuning().force_gemm_split > 0 ? tuning().force_gemm_split : kGemmMaxSplit;
+    int ks = knob(kGemmSplit) > 0 ? knob(kGemmSplit) : kGemmMaxSplit;
     if (ks > kGemmMaxSplit) ks = kGemmMaxSplit;
     if (ks > steps) ks = steps;
     if (ks < 1) ks = 1;
@@ -211,6 +277,93 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
         case 6: launch_gemm<6>(geo, x, qweight, lut, out, M, N, K, st); break;
         case 7: launch_gemm<7>(geo, x, qweight, lut, out, M, N, K, st); break;
         default: launch_gemm<8>(geo, x, qweight, lut, out, M, N, K, st); break;
+    }
+    return launch_status();
+}
+
+// The row-streaming GEMV serves rows of a multiple of 128 elements (16-byte plane loads), an even number
+// of rows (it walks row pairs and stores them as one dword) and up to 4 activation rows.
+bool gemvp_fits(const uint16_t *out, int M, int N, int K) {
+    const int W = K >> 5;
+    return M >= 1 && M <= kGemvpMaxM && (W & 3) == 0 && (N & 1) == 0 &&
+           (W + 127) / 128 <= kGemvpMaxSeg && (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+}
+
+int run_gemvp(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
+              int w_bits, hipStream_t st) {
+    GemvpGeometry geo;
+    const int W = K >> 5, pairs = N >> 1;
+    geo.S = (W + 127) / 128;
+    // As many workgroups as keep `gemv_stream_waves` waves on every CU, each walking the same number
+    // of row pairs (+-1): a grid a little smaller than the cap beats a ragged last round.
+    int wpc = knob(kGemvStreamWaves);
+    if (wpc < 1) wpc = 1;
+    long long cap = (long long)cu_count() * wpc / geo.S;
+    if (cap < 1) cap = 1;
+    const long long rounds = (pairs + cap - 1) / cap;
+    geo.grid = (int)((pairs + rounds - 1) / rounds);
+    switch (w_bits) {
+        case 3: launch_gemvp<3>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 4: launch_gemvp<4>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 5: launch_gemvp<5>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 6: launch_gemvp<6>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 7: launch_gemvp<7>(M, geo, x, qweight, lut, out, N, K, st); break;
+        default: launch_gemvp<8>(M, geo, x, qweight, lut, out, N, K, st); break;
+    }
+    return launch_status();
+}
+
+// The fine-grained row-pair GEMV serves rows of a multiple of 64 elements (8-byte plane loads), an even
+// number of rows and up to 4 activation rows.
+bool gemvf_fits(const uint16_t *out, int M, int N, int K) {
+    const int W = K >> 5;
+    return M >= 1 && M <= kGemvfMaxM && (W & 1) == 0 && (N & 1) == 0 &&
+           (W + 63) / 64 <= kGemvfMaxSeg && (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
+}
+
+int run_gemvf(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
+              int w_bits, hipStream_t st) {
+    GemvfGeometry geo;
+    geo.S = ((K >> 5) + 63) / 64;
+    geo.grid = N >> 1;
+    switch (w_bits) {
+        case 3: launch_gemvf<3>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 4: launch_gemvf<4>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 5: launch_gemvf<5>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 6: launch_gemvf<6>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 7: launch_gemvf<7>(M, geo, x, qweight, lut, out, N, K, st); break;
+        default: launch_gemvf<8>(M, geo, x, qweight, lut, out, N, K, st); break;
+    }
+    return launch_status();
+}
+
+// The persistent row-loop GEMV serves rows of a multiple of 64 elements (8-byte plane loads) and up to 4
+// activation rows.
+bool gemvr_fits(int M, int N, int K) {
+    const int W = K >> 5;
+    return M >= 1 && M <= kGemvrMaxM && (W & 1) == 0 && (W + 127) / 128 <= kGemvrMaxSeg;
+}
+
+int run_gemvr(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
+              int w_bits, hipStream_t st) {
+    GemvrGeometry geo;
+    geo.S = ((K >> 5) + 127) / 128;
+    // `gemv_persist_waves` waves per CU, every workgroup walking the same number of rows (+-1), at most 64
+    // (a single-wave workgroup parks one result per lane until its loop ends)
+    int wpc = knob(kGemvPersistWaves);
+    if (wpc < 1) wpc = 1;
+    long long cap = (long long)cu_count() * wpc / geo.S;
+    if (cap < 1) cap = 1;
+    long long rounds = (N + cap - 1) / cap;
+    if (rounds > 64) rounds = 64;
+    geo.grid = (int)((N + rounds - 1) / rounds);
+    switch (w_bits) {
+        case 3: launch_gemvr<3>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 4: launch_gemvr<4>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 5: launch_gemvr<5>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 6: launch_gemvr<6>(M, geo, x, qweight, lut, out, N, K, st); break;
+        case 7: launch_gemvr<7>(M, geo, x, qweight, lut, out, N, K, st); break;
+        default: launch_gemvr<8>(M, geo, x, qweight, lut, out, N, K, st); break;
     }
     return launch_status();
 }
@@ -232,7 +385,7 @@ int run_gemv4(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, u
         geo.rq = 2;
         // one word group per wave (with two row quads: 64 weights per lane, as in the dot-product kernel)
         // unless the row is so long that a workgroup could not hold its waves
-        int G = tuning().force_gemv4_groups > 0 ? tuning().force_gemv4_groups : 1;
+        int G = knob(kGemv4Groups) > 0 ? knob(kGemv4Groups) : 1;
         if (G != 1 && G != 2 && G != 4) G = 1;
         while (G < 4 && (W + 16 * G - 1) / (16 * G) > kGemv4MaxSeg) G *= 2;
         geo.G = G;
@@ -262,6 +415,7 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     if (rc != AP_OK) return rc;
     if (M < 1 || M > kGemmMaxM) return AP_EBATCH;
     if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
+    drain_stale_error();
     return run_gemm(x, qweight, lut, out, M, N, K, w_bits, static_cast<hipStream_t>(stream));
 }
 
@@ -288,11 +442,54 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
         mem.out[g] = out[g];
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
+    drain_stale_error();
     if (rc == AP_ELIMIT) {
         // a row longer than one workgroup of the dot-product kernel covers (65536 elements at M <= 2,
         // 32768 beyond): the MFMA kernel walks rows of any length
         for (int g = 0; g < count; g++) {
             const int r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
+            if (r != AP_OK) return r;
+        }
+        return AP_OK;
+    }
+    // Three more dot-product kernels (one linear per launch each), all with the same lookups and sums as
+    // gemv_kbit_kernel but a different split of the work over waves.  Measured on cold planes they stay
+    // within +-6 % of it on every 7B/8B/70B shape -- a launch is bound by its latency chain (dispatch,
+    // first loads, table staging, last compute, segment sums) and by what the memory system delivers to a
+    // burst of requests, not by the instruction count -- so mode 1 uses them only where they won by 3 % or
+    // more on two boxes, for single linears:
+    //  - row-streaming kernel (fewest waves and instructions): 3 bits at batch 1 on linears of >= 8192
+    //    rows of <= 4096 elements (gate/up of the 7B/8B models: 3-5 %), 3-4 bits at batch 2 on rows of
+    //    >= 8192 elements (10-14 %);
+    //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-8 bits at batch 1 on the
+    //    same wide linears (3-6 %), 6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %).
+    // Mode 2 of a knob forces its kernel wherever it fits (tests, sweeps); mode 0 switches it off.
+    const int persist_mode = knob(kGemvPersist), fine_mode = knob(kGemvFine), stream_mode = knob(kGemvStream);
+    enum { kDot, kPersist, kFine, kStream } pick = kDot;
+    bool fits_r = true, fits_f = true, fits_p = true;
+    for (int g = 0; g < count; g++) {
+        fits_r = fits_r && gemvr_fits(M, N[g], K);
+        fits_f = fits_f && gemvf_fits(out[g], M, N[g], K);
+        fits_p = fits_p && gemvp_fits(out[g], M, N[g], K);
+    }
+    if (persist_mode >= 2 && fits_r) {
+        pick = kPersist;  // never the default: measured slower than the others on every shape
+    } else if (fine_mode >= 2 && fits_f) {
+        pick = kFine;
+    } else if (stream_mode >= 2 && fits_p) {
+        pick = kStream;
+    } else if (count == 1) {
+        const bool wide = N[0] >= 8192 && K <= 4096;
+        if (stream_mode == 1 && fits_p && ((M == 1 && wide && w_bits == 3) || (M == 2 && K >= 8192 && w_bits <= 4)))
+            pick = kStream;
+        else if (fine_mode == 1 && fits_f && ((M == 1 && wide && w_bits >= 6) || (M == 4 && K >= 8192 && w_bits >= 6)))
+            pick = kFine;
+    }
+    if (pick != kDot) {
+        for (int g = 0; g < count; g++) {
+            const int r = pick == kPersist ? run_gemvr(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st)
+                          : pick == kFine  ? run_gemvf(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st)
+                                           : run_gemvp(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
             if (r != AP_OK) return r;
         }
         return AP_OK;
@@ -305,7 +502,7 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
     //  - 5..8 activation rows on wide linears (16 rows per workgroup) with rows of 3072..4096 elements
     //    (5..8 waves per workgroup): 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and longer
     //    rows and narrower linears measured slower.
-    const int m4 = tuning().mfma4_mode;
+    const int m4 = knob(kMatmulMfma4);
     long long rows = 0;
     for (int g = 0; g < count; g++) rows += N[g];
     auto use4 = [&](int n) {
@@ -332,7 +529,7 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
     }
     // From 5 activation rows on, the 16x16x32 MFMA kernel (cost flat in M up to 16 rows) is faster than
     // the dot-product kernel (cost linear in M) on most shapes and bit-widths; one linear per launch.
-    if (M >= tuning().mfma_from_rows) {
+    if (M >= knob(kMatmulMfmaFrom)) {
         for (int g = 0; g < count; g++) {
             const int r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
             if (r != AP_OK) return r;

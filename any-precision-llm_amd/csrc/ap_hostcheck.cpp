@@ -51,6 +51,28 @@ int aph_planes_to_nibbles(const uint32_t *q, int bits, uint32_t *nib) {
     return -1;
 }
 
+int aph_planes_to_adjacent_pairs(const uint32_t *q, int bits, uint32_t *apair) {
+    uint32_t out[4];
+    if (bits == 3) {
+        uint32_t qq[3] = {q[0], q[1], q[2]};
+        ap::planes_to_adjacent_pairs<3>(qq, out);
+    } else if (bits == 4) {
+        uint32_t qq[4] = {q[0], q[1], q[2], q[3]};
+        ap::planes_to_adjacent_pairs<4>(qq, out);
+    } else {
+        return -1;
+    }
+    for (int i = 0; i < 4; i++) apair[i] = out[i];
+    return 0;
+}
+
+int aph_adjacent_pair_split(int bits, uint32_t byte, uint32_t *first, uint32_t *second) {
+    if (bits == 3) ap::adjacent_pair_split<3>(byte, *first, *second);
+    else if (bits == 4) ap::adjacent_pair_split<4>(byte, *first, *second);
+    else return -1;
+    return 0;
+}
+
 int aph_chunk_words(int w, int K) { return ap::chunk_words(w, K); }
 int aph_group_base(int w, int j, int K) { return ap::group_base(w, j, K); }
 

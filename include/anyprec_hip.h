@@ -5,7 +5,9 @@
  * (any_precision/modules/kernels/main.cu).  Plain pointers and sizes only; all
  * pointers are device pointers on the current HIP device, all buffers are
  * owned by the caller, nothing is allocated or synchronised inside, and every
- * launch goes to the stream that is passed in (NULL = default stream).
+ * launch goes to the stream that is passed in (NULL = default stream).  The only
+ * state the library keeps is the table of tuning knobs behind ap_set_tuning and
+ * the CU count of each device, looked up on first use.
  *
  * Data formats (identical to the reference checkpoint format):
  *   qweight  uint32 [planes >= w_bits, N, K/32], contiguous; bit pattern of the
@@ -17,7 +19,10 @@
  *   x        fp16 [M, K] row-major;  out fp16 [M, N] (matmul) or [N, K] (dequant).
  *
  * Return value: AP_OK (0), a negative AP_E* argument error, or a positive
- * hipError_t from the launch.  The library never exits the process (the
+ * hipError_t from the launch (an error some earlier HIP call of the thread left
+ * behind is discarded, not reported).  An entry point that issues several launches
+ * (grouped linears, batches split in chunks) stops at the first one that fails: the
+ * outputs of the launches before it may already be written.  The library never exits the process (the
  * reference prints and calls exit(), main.cu:5-12).
  */
 #ifndef ANYPREC_HIP_H
@@ -29,7 +34,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 2
+#define AP_ABI_VERSION 3
 
 enum {
     AP_OK = 0,
@@ -38,7 +43,8 @@ enum {
     AP_ESHAPE = -3,  /* N < 1, K < 32 or K not a multiple of 32 (pack.py:15) */
     AP_EALIGN = -4,  /* a pointer is not 16-byte aligned                    */
     AP_EBATCH = -5,  /* M outside the range the entry point serves          */
-    AP_ELIMIT = -6   /* a size exceeds what the launch geometry can express */
+    AP_ELIMIT = -6,  /* a size exceeds what the launch geometry can express */
+    AP_EKNOB = -7    /* ap_set_tuning / ap_get_tuning: no knob of that name  */
 };
 
 /* Replaces dequant_kbit(qweight, lut, w_bits) -> Tensor[N,K]
@@ -58,8 +64,10 @@ int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *l
  * `count` device pointers / row counts.  For the q/k/v and gate/up projections of a decoder
  * layer, whose launches are otherwise bound by the fixed cost of a kernel launch.  No
  * counterpart in the reference (its hook for it, fuse_layers, is a stub:
- * AnyPrecisionForCausalLM.py:168-172); results equal `count` calls of ap_matmul_kbit bit
- * for bit.  1 <= M <= 8. */
+ * AnyPrecisionForCausalLM.py:168-172).  Results equal `count` calls of ap_matmul_kbit within
+ * the 1e-2 bar of the path, and bit for bit whenever the same kernel serves both (always with
+ * the tuning knobs gemv_stream and gemv_fine at 0: a few wide shapes otherwise go to a kernel
+ * that sums in another order when called one by one).  1 <= M <= 8. */
 int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight,
                          const uint16_t *const *lut, uint16_t *const *out, const int *N,
                          int M, int K, int w_bits, void *stream);
@@ -83,6 +91,25 @@ int ap_abi_version(void);
  * Returns AP_OK or the same argument errors as ap_matmul_kbit. */
 int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits,
                             int *wpl, int *segments, int *rows, int *grid);
+
+/* Test and measurement hook, no counterpart in the reference: overrides one launch-heuristic knob
+ * (which kernel variant serves a shape, grid sizes) for the whole process, so that tests can force
+ * every variant onto shapes they can check and benchmarks can sweep.  Results never depend on a knob
+ * beyond the 1e-2 bar of the entry points; the defaults are what measured fastest.  Names:
+ * gemv_target_waves, gemv_rows, gemv_wpl, dequant_blocks_per_cu, matmul_mfma_from, gemm_split,
+ * matmul_mfma4, gemv4_groups, gemm_rb2, gemv_stream, gemv_stream_waves, gemv_fine,
+ * gemv_persist, gemv_persist_waves.  Returns AP_OK, AP_ENULL or AP_EKNOB. */
+int ap_set_tuning(const char *name, int value);
+int ap_get_tuning(const char *name, int *value);
+
+/* Measurement aids, no counterpart in the reference.  ap_probe_stream only READS bytes0 bytes at buf0
+ * and bytes1 bytes at buf1 (multiples of 16; buf1 may be NULL with bytes1 = 0) with 16-byte non-temporal
+ * loads from `waves_per_cu` waves per CU (<= 0: 8) and writes nothing but possibly sink[0]: timed over
+ * the planes and tables of a linear it is the floor any kernel over those bytes has on this machine.
+ * ap_probe_empty launches one wave that does nothing: the fixed cost of a launch. */
+int ap_probe_stream(const void *buf0, long long bytes0, const void *buf1, long long bytes1,
+                    uint32_t *sink, int waves_per_cu, void *stream);
+int ap_probe_empty(uint32_t *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -42,7 +42,7 @@ def test_strerror_and_argument_errors_need_no_gpu():
     from any_precision_amd import _capi
     L = _capi.lib
     assert _capi.strerror(0) == "ok"
-    for code in (-1, -2, -3, -4, -5, -6):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert _capi.strerror(code) not in ("ok", "unknown error code")
     fake = 4096  # non-null, 16-byte aligned; argument errors return before any launch
     assert L.ap_dequant_kbit(None, fake, fake, 4, 64, 3, None) == _capi.AP_ENULL
@@ -73,3 +73,23 @@ def test_geometry_covers_rows_and_words():
             assert g["grid"] * g["rows"] >= N and (g["grid"] - 1) * g["rows"] < N
     with pytest.raises(ValueError):
         _capi.matmul_geometry(1, 4, 32 * 64 * 2 * 17, 4)     # more K-segments than a workgroup holds
+
+
+def test_tuning_knobs_need_no_gpu():
+    """ap_set_tuning / ap_get_tuning only touch the library's knob table."""
+    from any_precision_amd import _capi
+    assert _capi.lib.ap_set_tuning(None, 1) == _capi.AP_ENULL
+    assert _capi.lib.ap_set_tuning(b"no_such_knob", 1) == _capi.AP_EKNOB
+    with pytest.raises(ValueError):
+        _capi.get_tuning("no_such_knob")
+    for name in ("gemv_target_waves", "gemv_rows", "gemv_wpl", "dequant_blocks_per_cu", "matmul_mfma_from", "gemm_split",
+                 "matmul_mfma4", "gemv4_groups", "gemm_rb2", "gemv_stream", "gemv_stream_waves", "gemv_fine",
+                 "gemv_persist", "gemv_persist_waves"):
+        before = _capi.get_tuning(name)
+        with _capi.tuning(**{name: before + 3}):
+            assert _capi.get_tuning(name) == before + 3
+        assert _capi.get_tuning(name) == before
+    # the geometry report follows the knobs at once: nothing is cached
+    with _capi.tuning(gemv_rows=2):
+        assert _capi.matmul_geometry(1, 4096, 4096, 4)["rows"] == 2
+    assert _capi.matmul_geometry(1, 4096, 4096, 4)["rows"] == 1

@@ -125,47 +125,24 @@ def test_graph_replay_matches_eager(ext):
         assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), rep
 
 
-def test_two_weight_row_blocks_per_workgroup_give_the_same_bits(ext, oracle, tmp_path):
-    """Large linears run the MFMA kernel with two blocks of 16 weight rows per workgroup; AP_GEMM_RB2=2
-    (read once per process) forces that variant on the small ragged shapes a test can check against
-    the oracle.  Each output is still summed in the same order, so the results must equal the
-    one-block variant's bit for bit.  More than 32 activation rows go through it in chunks of 32."""
-    import os
-    import subprocess
-    import sys
+def test_two_weight_row_blocks_per_workgroup_give_the_same_bits(ext, oracle):
+    """Large linears run the MFMA kernel with two blocks of 16 weight rows per workgroup; the tuning knob
+    gemm_rb2 = 2 forces that variant on the small ragged shapes a test can check against the oracle.  Each
+    output is still summed in the same order, so the results must equal the one-block variant's bit for
+    bit.  More than 32 activation rows go through it in chunks of 32."""
+    from any_precision_amd import _capi
     shapes = ((33, 1024), (47, 2176), (130, 4096), (32, 128))
-    code = r"""
-import sys, torch
-sys.path[:0] = [%r, %r, %r]
-import oracle, any_precision_ext as ext
-from _util import assert_close_gemv, layer_to_gpu, make
-from any_precision_amd import synth
-res = {}
-for N, K in %r:
-    L = make(N, K, seed=N + K)
-    q, luts = layer_to_gpu(L)
-    for b in range(3, 9):
-        for M in (9, 16, 20, 32, 40, 100):
-            print(f"two row blocks N={N} K={K} b={b} M={M}", flush=True)
-            x = synth.make_x(M, K, seed=M)
-            got = ext.gemm_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
-            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
-            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
-            res[f"{N}_{K}_{b}_{M}"] = got.cpu()
-torch.save(res, %r)
-print("ok")
-"""
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = str(tmp_path / "forced.pt")
-    code = code % (root, os.path.join(root, "any-precision-llm_amd"), os.path.join(root, "tests"), shapes, out)
-    env = dict(os.environ, AP_GEMM_RB2="2")
-    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=280)
-    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), (r.stdout[-2000:], r.stderr[-2000:])
-    forced = torch.load(out, weights_only=True)
     for N, K in shapes:
         L = make(N, K, seed=N + K)
         q, luts = layer_to_gpu(L)
         for b in range(3, 9):
             for M in (9, 16, 20, 32, 40, 100):
-                _, xg = _x(M, K, seed=M)
-                assert torch.equal(ext.gemm_kbit(xg, q, luts[b], b).cpu(), forced[f"{N}_{K}_{b}_{M}"]), (N, K, b, M)
+                print(f"two row blocks N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                with _capi.tuning(gemm_rb2=2):
+                    forced = ext.gemm_kbit(xg, q, luts[b], b)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                assert_close_gemv(forced, want, f"N={N} K={K} b={b} M={M}")
+                with _capi.tuning(gemm_rb2=0):
+                    plain = ext.gemm_kbit(xg, q, luts[b], b)
+                assert torch.equal(plain.view(torch.int16), forced.view(torch.int16)), (N, K, b, M)

@@ -151,6 +151,10 @@ def test_graph_replay_matches_eager(ext):
 
 @pytest.mark.parametrize("K,Ns", [(4096, (512, 128, 128)), (1056, (33, 7, 64, 5)), (11008, (96, 96)), (96, (3,))])
 def test_group_launch_equals_separate_calls_bit_for_bit(ext, oracle, K, Ns):
+    """One launch for several linears: the same bits as one call per linear while the same kernel serves
+    both (the alternative dot-product kernels, which only single calls use, switched off), and the oracle's
+    values at the path's bar either way."""
+    from any_precision_amd import _capi
     layers = [make(N, K, seed=40 + i) for i, N in enumerate(Ns)]
     gpu = [layer_to_gpu(L) for L in layers]
     for b in (3, 4, 5, 8):
@@ -161,10 +165,12 @@ def test_group_launch_equals_separate_calls_bit_for_bit(ext, oracle, K, Ns):
             assert len(outs) == len(Ns)
             for (q, luts), L, got in zip(gpu, layers, outs):
                 assert got.shape == (M, L.N)
-                single = ext.matmul_kbit(xg, q, luts[b], b)
+                with _capi.tuning(gemv_stream=0, gemv_fine=0):
+                    single = ext.matmul_kbit(xg, q, luts[b], b)
                 assert torch.equal(got, single)
                 _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
                 assert_close_gemv(got, want, f"K={K} N={L.N} b={b} M={M}")
+                assert_close_gemv(ext.matmul_kbit(xg, q, luts[b], b), want, f"single K={K} N={L.N} b={b} M={M}")
 
 
 def test_group_argument_errors(ext):
@@ -181,37 +187,91 @@ def test_group_argument_errors(ext):
         ext.matmul_kbit_group(xg, [q, q2], [luts[3], luts2[3]], 3)    # different in_features
 
 
-def test_every_kernel_for_small_batches_agrees_with_the_oracle(oracle):
-    """ap_matmul_kbit picks between the dot-product kernel and the 4x4x4 matrix-core kernel by
-    shape and bit-width; AP_MATMUL_MFMA4 (read once per process) forces either, so each is run
-    in a child process on shapes the default rule would give to the other."""
-    import os
-    import subprocess
-    import sys
-    code = r"""
-import sys, numpy as np, torch
-sys.path[:0] = [%r, %r, %r]
-import oracle, any_precision_ext as ext
-from _util import assert_close_gemv, layer_to_gpu, make
-from any_precision_amd import synth
-for N, K in ((40, 2080), (2056, 1024), (9, 11008)):
-    L = make(N, K, seed=N)
+def test_every_kernel_for_small_batches_agrees_with_the_oracle(ext, oracle):
+    """ap_matmul_kbit picks between the dot-product kernel and the 4x4x4 matrix-core kernel by shape and
+    bit-width; the tuning knob matmul_mfma4 forces either (0 never, 2 wherever it fits), so each is run
+    on shapes the default rule would give to the other."""
+    from any_precision_amd import _capi
+    for N, K in ((40, 2080), (2056, 1024), (9, 11008)):
+        L = make(N, K, seed=N)
+        q, luts = layer_to_gpu(L)
+        for b in (3, 6, 8):
+            for M in (2, 3, 4, 5, 7, 8):
+                x, xg = _x(M, K, seed=M)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                for mode in (0, 2):
+                    print(f"forced kernel mfma4={mode} N={N} K={K} b={b} M={M}", flush=True)
+                    with _capi.tuning(matmul_mfma4=mode):
+                        got = ext.matmul_kbit(xg, q, luts[b], b)
+                    assert_close_gemv(got, want, f"mfma4={mode} N={N} K={K} b={b} M={M}")
+
+
+# (rows, elements per row): tails (K % 1024 != 0), one word group, one/several waves per row, many rows
+WAVE_SPLIT_SHAPES = [(2, 64), (130, 128), (34, 1088), (10, 2048), (64, 4096), (256, 11008), (20, 8192), (12, 14336),
+                     (6, 28672), (1030, 1024)]
+
+
+@pytest.mark.parametrize("knob", ["gemv_fine", "gemv_stream", "gemv_persist"])
+def test_the_other_splits_of_the_work_over_waves_agree_with_the_oracle(ext, oracle, knob):
+    """Three more dot-product kernels serve 1..4 activation rows (fine-grained row pairs, row-streaming
+    row pairs with 16-byte loads, persistent row loop); the default rule uses them on a few wide shapes
+    only, so each is forced (knob = 2) over ragged and tail shapes, every bit-width, M = 1..4, and checked
+    against the oracle at the path's 1e-2 bar.  Shapes a kernel does not serve (odd row counts, rows that
+    are not a multiple of 64 / 128 elements) must fall through to the default kernels."""
+    from any_precision_amd import _capi
+    for N, K in WAVE_SPLIT_SHAPES + [(7, 4096), (5, 96), (4, 2080)]:
+        L = make(N, K, seed=N + K)
+        q, luts = layer_to_gpu(L)
+        for b in range(3, 9):
+            for M in (1, 2, 3, 4):
+                print(f"{knob} N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                for waves in ((1, 24) if knob != "gemv_fine" else (0,)):
+                    extra = {knob + "_waves": waves} if waves else {}
+                    with _capi.tuning(**{knob: 2}, **extra):
+                        got = ext.matmul_kbit(xg, q, luts[b], b)
+                    assert_close_gemv(got, want, f"{knob} waves={waves} N={N} K={K} b={b} M={M}")
+
+
+@pytest.mark.parametrize("knob", ["gemv_fine", "gemv_stream", "gemv_persist"])
+def test_the_other_splits_are_exact_on_one_hot_activations_and_deterministic(ext, oracle, knob):
+    """x = e_k picks column k of the dequantised weight: the fp16 result must be that table entry bit for
+    bit (covers the word -> element mapping of every lane, tail chunk included); two runs must agree."""
+    from any_precision_amd import _capi
+    N, K = 66, 11008
+    L = make(N, K, seed=5)
     q, luts = layer_to_gpu(L)
-    for b in (3, 6, 8):
-        for M in (2, 3, 4, 5, 7, 8):
-            print(f"forced kernel N={N} K={K} b={b} M={M}", flush=True)
-            x = synth.make_x(M, K, seed=M)
-            got = ext.matmul_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
-            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
-            assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
-print("ok")
-"""
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    code = code % (root, os.path.join(root, "any-precision-llm_amd"), os.path.join(root, "tests"))
-    for mode in ("0", "2"):
-        env = dict(os.environ, AP_MATMUL_MFMA4=mode)
-        res = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=280)
-        assert res.returncode == 0 and res.stdout.strip().endswith("ok"), (mode, res.stdout[-2000:], res.stderr[-2000:])
+    for b in (3, 4, 5, 8):
+        w = oracle.dequant_kbit(L.qweight, L.luts[b], b)
+        for k in (0, 7, 8, 255, 256, 1023, 1024, 4095, 4096, 10239, 10240, 10431, 10432, 11007):
+            x = np.zeros((1, K), dtype=np.float16)
+            x[0, k] = 1.0
+            with _capi.tuning(**{knob: 2}):
+                got = ext.matmul_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
+            assert_bit_exact(got, w[:, k].reshape(1, N), f"{knob} b={b} k={k}")
+        x, xg = _x(3, K, seed=b)
+        with _capi.tuning(**{knob: 2}):
+            first = ext.matmul_kbit(xg, q, luts[b], b)
+            again = ext.matmul_kbit(xg, q, luts[b], b)
+        assert torch.equal(first.view(torch.int16), again.view(torch.int16))
+
+
+def test_default_routing_on_wide_linears_agrees_with_the_oracle(ext, oracle):
+    """The shapes on which the default rule leaves the first dot-product kernel (gate/up projections of
+    the 7B/8B models at 3 and 6..8 bits, long rows at batch 2 and 4), against the oracle on a row slice."""
+    for N, K, Ms in ((11008, 4096, (1,)), (8192, 8192, (2, 4))):
+        L = make(N, K, seed=N)
+        q, luts = layer_to_gpu(L)
+        for b in (3, 4, 6, 8):
+            for M in Ms:
+                print(f"default route N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                got = ext.matmul_kbit(xg, q, luts[b], b)
+                rows = slice(N - 300, N)
+                _, want = oracle.matmul_kbit(x, np.ascontiguousarray(L.qweight[:, rows]), L.luts[b][rows], b, return_f64=True)
+                assert_close_gemv(got[:, rows], want, f"N={N} K={K} b={b} M={M}")
+
 
 
 def test_rows_longer_than_a_workgroup_covers(ext):

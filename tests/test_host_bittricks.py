@@ -50,6 +50,31 @@ def test_pair_indices(hostcheck, oracle, bits):
         assert np.array_equal(out, oracle.transpose_pair(q, bits) << np.uint32(shift))
 
 
+@pytest.mark.parametrize("bits", [3, 4])
+def test_adjacent_pair_indices(hostcheck, oracle, bits):
+    """Byte b of apair[i] names the table entry of elements (2i, 2i+1) of byte group 3 - b: splitting it
+    must give back the two indices the oracle's transpose holds for those elements (idx[e] byte b)."""
+    rng = np.random.default_rng(70 + bits)
+    first, second = ctypes.c_uint32(), ctypes.c_uint32()
+    for trial in range(200):
+        q = rng.integers(0, 2**32, size=bits, dtype=np.uint64).astype(np.uint32)
+        if trial < bits * 2:                 # walking planes: all ones / a single one
+            q = np.zeros(bits, dtype=np.uint32)
+            q[trial % bits] = np.uint32(0xFFFFFFFF if trial < bits else 1 << (5 * trial % 32))
+        out = np.zeros(4, dtype=np.uint32)
+        assert hostcheck.aph_planes_to_adjacent_pairs(ctypes.c_void_p(q.ctypes.data), bits,
+                                                      ctypes.c_void_p(out.ctypes.data)) == 0
+        want = oracle.transpose(q, bits)     # want[e] byte b = index of element e of that byte
+        for i in range(4):
+            for b in range(4):
+                byte = (int(out[i]) >> (8 * b)) & 0xFF
+                if bits == 3:
+                    assert byte % 4 == 0     # a dword offset into 64 entries
+                assert hostcheck.aph_adjacent_pair_split(bits, byte, ctypes.byref(first), ctypes.byref(second)) == 0
+                assert first.value == (int(want[2 * i]) >> (8 * b)) & 0xFF, (i, b)
+                assert second.value == (int(want[2 * i + 1]) >> (8 * b)) & 0xFF, (i, b)
+
+
 @pytest.mark.parametrize("bits", [1, 2, 3, 4])
 def test_nibble_indices(hostcheck, oracle, bits):
     rng = np.random.default_rng(60 + bits)
