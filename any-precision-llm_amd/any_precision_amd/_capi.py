@@ -43,6 +43,8 @@ lib.ap_probe_stream.argtypes = [_vp, ctypes.c_longlong, _vp, ctypes.c_longlong, 
 lib.ap_probe_stream.restype = _ci
 lib.ap_probe_empty.argtypes = [_vp, _vp]
 lib.ap_probe_empty.restype = _ci
+lib.ap_matmul_kbit_route.argtypes = [_ci, _ci, _ci, _ci, _pi]
+lib.ap_matmul_kbit_route.restype = _ci
 lib.ap_set_tuning.argtypes = [ctypes.c_char_p, _ci]
 lib.ap_set_tuning.restype = _ci
 lib.ap_get_tuning.argtypes = [ctypes.c_char_p, _pi]
@@ -54,7 +56,7 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
     )
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
-           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty")
+           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_matmul_kbit_route")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
 
@@ -84,6 +86,16 @@ def matmul_geometry(M: int, N: int, K: int, w_bits: int) -> dict:
     vals = [ctypes.c_int() for _ in range(4)]
     check(lib.ap_matmul_kbit_geometry(M, N, K, w_bits, *[ctypes.byref(v) for v in vals]), "ap_matmul_kbit_geometry")
     return dict(zip(("wpl", "segments", "rows", "grid"), (v.value for v in vals)))
+
+
+ROUTES = ("dot", "stream", "fine", "persist", "mfma4", "mfma16")
+
+
+def matmul_route(M: int, N: int, K: int, w_bits: int) -> str:
+    """Name of the kernel ap_matmul_kbit launches for one linear of this shape."""
+    r = ctypes.c_int()
+    check(lib.ap_matmul_kbit_route(M, N, K, w_bits, ctypes.byref(r)), "ap_matmul_kbit_route")
+    return ROUTES[r.value]
 
 
 def set_tuning(name: str, value: int) -> None:

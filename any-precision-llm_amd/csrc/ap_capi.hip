@@ -315,7 +315,7 @@ int run_gemvp(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, u
 
 // The fine-grained row-pair GEMV serves rows of a multiple of 64 elements (8-byte plane loads), an even
 // number of rows and up to 4 activation rows.
-bool gemvf_fits(const uint16_t *out, int M, int N, int K) {
+bool gemvf_fits(const uint16_t *out, int M, int N, int K) {  // out == nullptr: taken to be aligned
     const int W = K >> 5;
     return M >= 1 && M <= kGemvfMaxM && (W & 1) == 0 && (N & 1) == 0 &&
            (W + 63) / 64 <= kGemvfMaxSeg && (reinterpret_cast<uintptr_t>(out) & 3u) == 0;
@@ -404,6 +404,85 @@ int run_gemv4(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, u
     return launch_status();
 }
 
+// Which kernel serves each of `count` linears that share x, M, K and w_bits (route[g] = AP_ROUTE_*), and the
+// geometry of the grouped dot-product launch when that is the answer (then every member has AP_ROUTE_DOT).
+// `out` may be null (route queries): the output pointers are then taken to be aligned.
+int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *const *out, GemvGeometry *geo,
+                GemvMembers *mem, int *route) {
+    const int rc = gemv_geometry(M, N, count, K, w_bits, geo, mem);
+    if (rc != AP_OK && rc != AP_ELIMIT) return rc;
+    auto all = [&](int r) {
+        for (int g = 0; g < count; g++) route[g] = r;
+        return AP_OK;
+    };
+    // a row longer than one workgroup of the dot-product kernel covers (65536 elements at M <= 2, 32768
+    // beyond): the MFMA kernel walks rows of any length
+    if (rc == AP_ELIMIT) return all(AP_ROUTE_MFMA16);
+    // Three more dot-product kernels (one linear per launch each), all with the same lookups and sums as
+    // gemv_kbit_kernel but a different split of the work over waves.  Measured on cold planes they stay
+    // within +-6 % of it on every 7B/8B/70B shape -- a launch is bound by its latency chain (dispatch,
+    // first loads, table staging, last compute, segment sums) and by what the memory system delivers to a
+    // burst of requests, not by the instruction count -- so mode 1 uses them only where they won by 3 % or
+    // more on two boxes, for single linears:
+    //  - row-streaming kernel (fewest waves and instructions): 3 bits at batch 1 on linears of >= 8192
+    //    rows of <= 4096 elements (gate/up of the 7B/8B models: 3-5 %), 3-4 bits at batch 2 on rows of
+    //    >= 8192 elements (10-14 %);
+    //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-8 bits at batch 1 on the
+    //    same wide linears (3-6 %), 6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %).
+    // Mode 2 of a knob forces its kernel wherever it fits (tests, sweeps); mode 0 switches it off.
+    const int persist_mode = knob(kGemvPersist), fine_mode = knob(kGemvFine), stream_mode = knob(kGemvStream);
+    bool fits_r = true, fits_f = true, fits_p = true;
+    for (int g = 0; g < count; g++) {
+        const uint16_t *o = out ? out[g] : nullptr;
+        fits_r = fits_r && gemvr_fits(M, N[g], K);
+        fits_f = fits_f && gemvf_fits(o, M, N[g], K);
+        fits_p = fits_p && gemvp_fits(o, M, N[g], K);
+    }
+    if (persist_mode >= 2 && fits_r) return all(AP_ROUTE_PERSIST);  // never the default: slower on every shape
+    if (fine_mode >= 2 && fits_f) return all(AP_ROUTE_FINE);
+    if (stream_mode >= 2 && fits_p) return all(AP_ROUTE_STREAM);
+    if (count == 1) {
+        const bool wide = N[0] >= 8192 && K <= 4096;
+        if (stream_mode == 1 && fits_p && ((M == 1 && wide && w_bits == 3) || (M == 2 && K >= 8192 && w_bits <= 4)))
+            return all(AP_ROUTE_STREAM);
+        if (fine_mode == 1 && fits_f && ((M == 1 && wide && w_bits >= 6) || (M == 4 && K >= 8192 && w_bits >= 6)))
+            return all(AP_ROUTE_FINE);
+    }
+    // The 4x4x4 matrix-core kernel, whose cost per weight does not grow with M, where it measured
+    // faster than both other kernels (it serves one linear per launch):
+    //  - 3 and 4 activation rows on linears with enough rows to fill the chip (8 per workgroup), at up
+    //    to 5 bits, and for 4 rows at every bit-width while a row fits one word group per lane
+    //    (K <= 8192): 10-40 % faster than the dot-product kernel;
+    //  - 5..8 activation rows on wide linears (16 rows per workgroup) with rows of 3072..4096 elements
+    //    (5..8 waves per workgroup): 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and longer
+    //    rows and narrower linears measured slower.
+    const int m4 = knob(kMatmulMfma4);
+    long long rows = 0;
+    for (int g = 0; g < count; g++) rows += N[g];
+    auto use4 = [&](int n) {
+        const int W = K >> 5;
+        if (m4 == 0 || M < 2 || M > 8) return false;
+        if (M <= 4) {  // decided for the group as a whole, by its mean row count
+            if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
+            if (m4 >= 2) return true;
+            return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192))) && rows >= 2048LL * count;
+        }
+        if (W > 16 * kGemv4MaxSegTwo) return false;
+        if (m4 >= 2) return true;
+        return K >= 3072 && n >= 10240;  // per member; the others go to the MFMA kernel
+    };
+    bool any4 = false;
+    for (int g = 0; g < count; g++) any4 |= use4(N[g]);
+    if (any4) {
+        for (int g = 0; g < count; g++) route[g] = use4(N[g]) ? AP_ROUTE_MFMA4 : AP_ROUTE_MFMA16;
+        return AP_OK;
+    }
+    // From 5 activation rows on, the 16x16x32 MFMA kernel (cost flat in M up to 16 rows) is faster than
+    // the dot-product kernel (cost linear in M) on most shapes and bit-widths; one linear per launch.
+    if (M >= knob(kMatmulMfmaFrom)) return all(AP_ROUTE_MFMA16);
+    return all(AP_ROUTE_DOT);
+}
+
 }  // namespace
 
 extern "C" {
@@ -432,8 +511,9 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
         if (!qweight[g] || !lut[g] || !out[g]) return AP_ENULL;
     GemvGeometry geo;
     GemvMembers mem = {};
-    const int rc = gemv_geometry(M, N, count, K, w_bits, &geo, &mem);
-    if (rc != AP_OK && rc != AP_ELIMIT) return rc;
+    int route[kGemvMaxGroup];
+    const int rc = plan_matmul(M, N, count, K, w_bits, out, &geo, &mem, route);
+    if (rc != AP_OK) return rc;
     if (!aligned16(x)) return AP_EALIGN;
     for (int g = 0; g < count; g++) {
         if (!aligned16(qweight[g]) || !aligned16(lut[g])) return AP_EALIGN;
@@ -443,108 +523,35 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     drain_stale_error();
-    if (rc == AP_ELIMIT) {
-        // a row longer than one workgroup of the dot-product kernel covers (65536 elements at M <= 2,
-        // 32768 beyond): the MFMA kernel walks rows of any length
-        for (int g = 0; g < count; g++) {
-            const int r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
-            if (r != AP_OK) return r;
+    if (route[0] == AP_ROUTE_DOT) {  // the whole set in one launch (plan_matmul gives all members this route or none)
+        switch (w_bits) {
+            case 3: launch_gemv<3>(M, geo, x, mem, K, st); break;
+            case 4: launch_gemv<4>(M, geo, x, mem, K, st); break;
+            case 5: launch_gemv<5>(M, geo, x, mem, K, st); break;
+            case 6: launch_gemv<6>(M, geo, x, mem, K, st); break;
+            case 7: launch_gemv<7>(M, geo, x, mem, K, st); break;
+            default: launch_gemv<8>(M, geo, x, mem, K, st); break;
         }
-        return AP_OK;
+        return launch_status();
     }
-    // Three more dot-product kernels (one linear per launch each), all with the same lookups and sums as
-    // gemv_kbit_kernel but a different split of the work over waves.  Measured on cold planes they stay
-    // within +-6 % of it on every 7B/8B/70B shape -- a launch is bound by its latency chain (dispatch,
-    // first loads, table staging, last compute, segment sums) and by what the memory system delivers to a
-    // burst of requests, not by the instruction count -- so mode 1 uses them only where they won by 3 % or
-    // more on two boxes, for single linears:
-    //  - row-streaming kernel (fewest waves and instructions): 3 bits at batch 1 on linears of >= 8192
-    //    rows of <= 4096 elements (gate/up of the 7B/8B models: 3-5 %), 3-4 bits at batch 2 on rows of
-    //    >= 8192 elements (10-14 %);
-    //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-8 bits at batch 1 on the
-    //    same wide linears (3-6 %), 6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %).
-    // Mode 2 of a knob forces its kernel wherever it fits (tests, sweeps); mode 0 switches it off.
-    const int persist_mode = knob(kGemvPersist), fine_mode = knob(kGemvFine), stream_mode = knob(kGemvStream);
-    enum { kDot, kPersist, kFine, kStream } pick = kDot;
-    bool fits_r = true, fits_f = true, fits_p = true;
     for (int g = 0; g < count; g++) {
-        fits_r = fits_r && gemvr_fits(M, N[g], K);
-        fits_f = fits_f && gemvf_fits(out[g], M, N[g], K);
-        fits_p = fits_p && gemvp_fits(out[g], M, N[g], K);
-    }
-    if (persist_mode >= 2 && fits_r) {
-        pick = kPersist;  // never the default: measured slower than the others on every shape
-    } else if (fine_mode >= 2 && fits_f) {
-        pick = kFine;
-    } else if (stream_mode >= 2 && fits_p) {
-        pick = kStream;
-    } else if (count == 1) {
-        const bool wide = N[0] >= 8192 && K <= 4096;
-        if (stream_mode == 1 && fits_p && ((M == 1 && wide && w_bits == 3) || (M == 2 && K >= 8192 && w_bits <= 4)))
-            pick = kStream;
-        else if (fine_mode == 1 && fits_f && ((M == 1 && wide && w_bits >= 6) || (M == 4 && K >= 8192 && w_bits >= 6)))
-            pick = kFine;
-    }
-    if (pick != kDot) {
-        for (int g = 0; g < count; g++) {
-            const int r = pick == kPersist ? run_gemvr(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st)
-                          : pick == kFine  ? run_gemvf(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st)
-                                           : run_gemvp(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
-            if (r != AP_OK) return r;
+        int r;
+        switch (route[g]) {
+            case AP_ROUTE_STREAM: r = run_gemvp(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
+            case AP_ROUTE_FINE: r = run_gemvf(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
+            case AP_ROUTE_PERSIST: r = run_gemvr(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
+            case AP_ROUTE_MFMA4: r = run_gemv4(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
+            default: r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
         }
-        return AP_OK;
+        if (r != AP_OK) return r;
     }
-    // The 4x4x4 matrix-core kernel, whose cost per weight does not grow with M, where it measured
-    // faster than both other kernels (it serves one linear per launch):
-    //  - 3 and 4 activation rows on linears with enough rows to fill the chip (8 per workgroup), at up
-    //    to 5 bits, and for 4 rows at every bit-width while a row fits one word group per lane
-    //    (K <= 8192): 10-40 % faster than the dot-product kernel;
-    //  - 5..8 activation rows on wide linears (16 rows per workgroup) with rows of 3072..4096 elements
-    //    (5..8 waves per workgroup): 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and longer
-    //    rows and narrower linears measured slower.
-    const int m4 = knob(kMatmulMfma4);
-    long long rows = 0;
-    for (int g = 0; g < count; g++) rows += N[g];
-    auto use4 = [&](int n) {
-        const int W = K >> 5;
-        if (m4 == 0 || M < 2 || M > 8) return false;
-        if (M <= 4) {  // decided for the group as a whole, by its mean row count
-            if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
-            if (m4 >= 2) return true;
-            return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192))) && rows >= 2048LL * count;
-        }
-        if (W > 16 * kGemv4MaxSegTwo) return false;
-        if (m4 >= 2) return true;
-        return K >= 3072 && n >= 10240;  // per member; the others go to the MFMA kernel
-    };
-    bool any4 = false;
-    for (int g = 0; g < count; g++) any4 |= use4(N[g]);
-    if (any4) {
-        for (int g = 0; g < count; g++) {
-            const int r = use4(N[g]) ? run_gemv4(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st)
-                                     : run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
-            if (r != AP_OK) return r;
-        }
-        return AP_OK;
-    }
-    // From 5 activation rows on, the 16x16x32 MFMA kernel (cost flat in M up to 16 rows) is faster than
-    // the dot-product kernel (cost linear in M) on most shapes and bit-widths; one linear per launch.
-    if (M >= knob(kMatmulMfmaFrom)) {
-        for (int g = 0; g < count; g++) {
-            const int r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st);
-            if (r != AP_OK) return r;
-        }
-        return AP_OK;
-    }
-    switch (w_bits) {
-        case 3: launch_gemv<3>(M, geo, x, mem, K, st); break;
-        case 4: launch_gemv<4>(M, geo, x, mem, K, st); break;
-        case 5: launch_gemv<5>(M, geo, x, mem, K, st); break;
-        case 6: launch_gemv<6>(M, geo, x, mem, K, st); break;
-        case 7: launch_gemv<7>(M, geo, x, mem, K, st); break;
-        default: launch_gemv<8>(M, geo, x, mem, K, st); break;
-    }
-    return launch_status();
+    return AP_OK;
+}
+
+int ap_matmul_kbit_route(int M, int N, int K, int w_bits, int *route) {
+    if (!route) return AP_ENULL;
+    GemvGeometry geo;
+    return plan_matmul(M, &N, 1, K, w_bits, nullptr, &geo, nullptr, route);
 }
 
 }  // extern "C"

@@ -66,12 +66,12 @@ class WeightPool:
     uniform plane bits, so planes are drawn directly as random words; tables are ascending
     N(0, 0.02) draws (std 0.02), one per set and precision."""
 
-    def __init__(self, torch, N, K, sets, gen):
+    def __init__(self, torch, N, K, sets, gen, bits=BITS):
         self.N, self.K, self.sets = N, K, sets
         self.qweight = torch.randint(-2**31, 2**31 - 1, (sets, 8, N, K // 32), dtype=torch.int32, device="cuda",
                                      generator=gen)
         self.luts = {}
-        for b in BITS:
+        for b in bits:
             t = torch.randn((sets, N, 1 << b), device="cuda", generator=gen) * 0.02
             self.luts[b] = torch.sort(t, dim=2).values.to(torch.float16).contiguous()
         self.out = torch.empty((8, N), dtype=torch.float16, device="cuda")
@@ -129,6 +129,17 @@ def main():
         j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
         rc = (fn or lib.ap_matmul_kbit)(xb[(M, K)].data_ptr(), P.qweight[j].data_ptr(), P.luts[b][j].data_ptr(),
                                         P.out.data_ptr(), M, N, K, b, stream)
+        if rc != 0:
+            raise RuntimeError(_capi.strerror(rc))
+
+    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
+
+    def read_only(N: int, K: int, b: int, stream: int):
+        """ap_probe_stream over the planes 0..b-1 and the table of the next weight set of the shape."""
+        P = pools[(N, K)]
+        j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
+        rc = lib.ap_probe_stream(P.qweight[j].data_ptr(), b * N * K // 8, P.luts[b][j].data_ptr(), N * (2 << b),
+                                 sink.data_ptr(), 32, stream)
         if rc != 0:
             raise RuntimeError(_capi.strerror(rc))
 
@@ -253,11 +264,16 @@ def main():
                 us_warm = time_graph(lambda st: lib.ap_matmul_kbit(xb[(1, K)].data_ptr(), P0.qweight[0].data_ptr(),
                                                                    P0.luts[b][0].data_ptr(), P0.out.data_ptr(), 1, N, K,
                                                                    b, st), args.kernel_reps)
+                # a kernel that only READS the same planes and tables (16-byte loads, no arithmetic, no
+                # output), launched over the same rotating pool: what the machine does for these bytes
+                us_read = time_graph(lambda st: read_only(N, K, b, st), reps)
                 table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 3), "us_min": round(lo, 3),
                               "us_max": round(hi, 3), "us_cache_resident": round(us_warm, 3),
+                              "stream_only_us": round(us_read, 3),
+                              "frac_of_stream_ceiling": round(us_read / us, 4),
                               "GBps": round(by / us / 1e3, 1),
                               "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4), "bytes": by,
-                              "count_in_step": len(idxs), "geometry": geo})
+                              "count_in_step": len(idxs), "kernel": _capi.matmul_route(1, N, K, b), "geometry": geo})
 
     # ---- further kernels of the path (reported beside the headline, not part of `value`)
     if not args.only_step and not args.no_extras:
@@ -290,6 +306,58 @@ def main():
                     row[f"us_M{M}"] = round(time_graph(lambda st: launch(N, K, b, st, M, fn), 24), 2)
                 batch_table.append(row)
 
+    # ---- compact figures for the other configurations (each has a --workload of its own with the full
+    # tables): the Llama-3-8B shapes at M = 1, 2, 4, 8 and dequant_kbit over a whole Llama-2-7B layer set
+    llama3, dequant_layer = None, None
+    if not args.only_step and not args.no_extras and not args.eager:
+        llama3 = []
+        for (N, K) in ((1024, 4096), (14336, 4096), (4096, 14336)):
+            sets = max(3, int(0.6e9 / (3 * N * K / 8)) + 1)
+            P3 = WeightPool(torch, N, K, sets, gen, bits=(3, 8))
+            cur = {"j": 0}
+            for b in (3, 8):
+                row = {"N": N, "K": K, "w_bits": b}
+                for M in (1, 2, 4, 8):
+                    x3 = xb[(M, 4096)] if K == 4096 else torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+                    out3 = torch.empty((M, N), dtype=torch.float16, device="cuda")
+
+                    def call3(st):
+                        cur["j"] = (cur["j"] + 1) % P3.sets
+                        rc = lib.ap_matmul_kbit(x3.data_ptr(), P3.qweight[cur["j"]].data_ptr(), P3.luts[b][cur["j"]].data_ptr(),
+                                                out3.data_ptr(), M, N, K, b, st)
+                        if rc != 0:
+                            raise RuntimeError(_capi.strerror(rc))
+                    us = time_graph(call3, min(24, 2 * sets))
+                    row[f"us_M{M}"] = round(us, 2)
+                    row[f"frac_M{M}"] = round(synth.gemv_bytes(N, K, b, M) / us / 1e3 / HBM_PEAK_GBS, 4)
+                llama3.append(row)
+            del P3
+            torch.cuda.empty_cache()
+        # dequant_kbit of the 7 linears of a layer, outputs rotating over >= 512 MB per shape: bytes read + written
+        # over time, per w_bits -- 32 such layer sets are the full model (configuration 4)
+        outs = {(N, K): [torch.empty((N, K), dtype=torch.float16, device="cuda")
+                         for _ in range(max(2, int(512e6 / (2 * N * K)) + 1))] for (N, K) in pools}
+        oi = {k: 0 for k in pools}
+
+        def dequant_layer_set(st, b):
+            for _, N, K in shapes:
+                P = pools[(N, K)]
+                j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
+                oi[(N, K)] = (oi[(N, K)] + 1) % len(outs[(N, K)])
+                rc = lib.ap_dequant_kbit(P.qweight[j].data_ptr(), P.luts[b][j].data_ptr(), outs[(N, K)][oi[(N, K)]].data_ptr(),
+                                         N, K, b, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+        dequant_layer = []
+        for b in BITS:
+            us = time_graph(lambda st: dequant_layer_set(st, b), 4)
+            by = sum(synth.dequant_bytes(N, K, b) for _, N, K in shapes)
+            dequant_layer.append({"w_bits": b, "us_per_layer_set": round(us, 1), "GBps": round(by / us / 1e3, 1),
+                                  "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
+                                  "full_model_ms": round(32 * us / 1e3, 3)})
+        del outs
+        torch.cuda.empty_cache()
+
     # ---- what this box gives a trivial kernel, in this run: a plain device copy (read 512 MiB + write
     # 512 MiB per launch) and an elementwise op on one element (the fixed cost of a graph node)
     machine = None
@@ -299,9 +367,26 @@ def main():
         us_copy = time_graph(lambda st: dst.copy_(src), 4)
         one = torch.zeros(1, device="cuda")
         us_node = time_graph(lambda st: one.add_(1.0), 200)
+        us_empty = time_graph(lambda st: lib.ap_probe_empty(sink.data_ptr(), st), 200)
+        # the GEMV itself with nothing to stream: 64 rows of 4096 elements (launch + first loads + table
+        # staging + lookups of one word per lane + reduction + store), the fixed cost every launch carries
+        P0 = pools[(4096, 4096)]
+        fixed = {}
+        for b in (3, 8):
+            fixed[f"w{b}"] = round(time_graph(
+                lambda st: lib.ap_matmul_kbit(xb[(1, 4096)].data_ptr(), P0.qweight[0].data_ptr(), P0.luts[b][0].data_ptr(),
+                                              P0.out.data_ptr(), 1, 64, 4096, b, st), 100), 3)
         machine = {"copy_GBps": round(2 * src.numel() * 4 / us_copy / 1e3, 1), "copy_bytes": 2 * src.numel() * 4,
-                   "graph_node_us": round(us_node, 3),
-                   "note": "torch copy of 512 MiB (read + write) and a 1-element add, both as HIP-graph nodes"}
+                   "graph_node_us": round(us_node, 3), "empty_kernel_us": round(us_empty, 3),
+                   "gemv_64_rows_us": fixed,
+                   "note": "torch copy of 512 MiB (read + write), a 1-element add, an empty kernel and the GEMV on 64 "
+                           "rows (whose planes are not 64 rows of a real layer but the first rows of one: same "
+                           "launch, nothing to stream), all as HIP-graph nodes"}
+        if table:
+            read_ms = sum(r["stream_only_us"] * r["count_in_step"] for r in table) / 1e3
+            machine["stream_only_step_ms"] = round(read_ms, 5)
+            machine["stream_only_GBps"] = round(step_bytes / read_ms / 1e6, 1)
+            machine["value_over_stream_only"] = round(read_ms / ms_per_step, 4)
         del src, dst
 
     roofline = None
@@ -315,63 +400,16 @@ def main():
                 traffic = json.load(f)["bytes"].get(f"{dom['N']}x{dom['K']}:{dom['w_bits']}")
         roofline = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": dom["frac"], "traffic": traffic,
-                    "kernel": f"gemv_kbit_kernel<{dom['w_bits']},1,{dom['geometry']['wpl']},*> {dom['N']}x{dom['K']}",
+                    "kernel": (f"gemv_kbit_kernel<{dom['w_bits']},1,{dom['geometry']['wpl']},*>" if dom["kernel"] == "dot"
+                               else f"{dom['kernel']} kernel, w_bits {dom['w_bits']}") + f" {dom['N']}x{dom['K']}",
+                    "stream_only_us": dom["stream_only_us"], "frac_of_stream_ceiling": dom["frac_of_stream_ceiling"],
                     "us_per_launch": dom["us"], "algorithmic_bytes_per_launch": dom["bytes"]}
 
-    # ---- CPU baseline: the oracle's host-speed GEMV (unpack + gather + dot), same shapes
+    # ---- CPU baseline: the oracle's host-speed GEMV (unpack + gather + dot), and the reference semantics
+    # written with PyTorch CPU ops, both timed on this box's host cores
     cpu = None
     if not args.no_cpu:
-        import numpy as np
-        import oracle
-        oracle.build()
-        rng = np.random.default_rng(0)
-        cpu_bits = (3, 8)
-        t_cpu, b_cpu = 0.0, 0
-        for _, N, K in [shapes[0], shapes[4], shapes[6]]:
-            qw = rng.integers(-2**31, 2**31 - 1, size=(8, N, K // 32), dtype=np.int64).astype(np.int32)
-            x = rng.normal(0, 1, size=(1, K)).astype(np.float16)
-            for b in cpu_bits:
-                lut = np.sort(rng.normal(0, 0.02, size=(N, 1 << b)), axis=1).astype(np.float16)
-                oracle.matmul_kbit_fast(x, qw, lut, b)                  # warm
-                reps, t0 = 0, time.perf_counter()
-                while reps < 3 or time.perf_counter() - t0 < 1.5:       # about 1.5 s per case, 10 s in all
-                    oracle.matmul_kbit_fast(x, qw, lut, b)
-                    reps += 1
-                t_cpu += (time.perf_counter() - t0) / reps
-                b_cpu += synth.gemv_bytes(N, K, b, 1)
-        cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
-               "sample": "C oracle GEMV (unpack+gather+fp32 dot, OpenMP over rows): 4096x4096, 11008x4096, "
-                         "4096x11008 at w_bits 3 and 8, batch 1, each repeated for about 1.5 s (mean)"}
-        # the same semantics written with PyTorch CPU ops (bitplane unpack -> table gather -> matmul), 4096x4096
-        N = K = 4096
-        nthr = torch.get_num_threads()
-        qw_t = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(8, N, K // 32), dtype=np.int64).astype(np.int32))
-        x_t = torch.from_numpy(rng.normal(0, 1, size=(1, K)).astype(np.float32))
-
-        def torch_unpack(b):
-            by = qw_t[:b].contiguous().view(torch.uint8).view(b, N, K // 1024, 32, 4).flip(-1)        # [p,n,c,t,j]
-            bits = (by.unsqueeze(-1) >> torch.arange(7, -1, -1, dtype=torch.uint8)) & 1                  # [p,n,c,t,j,e]
-            bits = bits.permute(0, 1, 2, 4, 3, 5).reshape(b, N, K)
-            w = (1 << torch.arange(b - 1, -1, -1, dtype=torch.int64)).view(b, 1, 1)
-            return (bits.to(torch.int64) * w).sum(0)
-
-        t_e2e, t_mm, by_t = 0.0, 0.0, 0
-        for b in cpu_bits:
-            lut_t = torch.from_numpy(np.sort(rng.normal(0, 0.02, size=(N, 1 << b)), axis=1).astype(np.float32))
-            t0 = time.perf_counter()
-            wdq = torch.gather(lut_t, 1, torch_unpack(b))
-            y = x_t @ wdq.T
-            t_e2e += time.perf_counter() - t0
-            t0 = time.perf_counter()
-            for _ in range(5):
-                y = x_t @ wdq.T
-            t_mm += (time.perf_counter() - t0) / 5
-            by_t += synth.gemv_bytes(N, K, b, 1)
-        cpu["torch_reference_semantics"] = {
-            "GBps_end_to_end": round(by_t / t_e2e / 1e9, 4), "ms_end_to_end": round(t_e2e * 1e3 / len(cpu_bits), 1),
-            "ms_matmul_only": round(t_mm * 1e3 / len(cpu_bits), 3), "threads": nthr,
-            "sample": "torch CPU ops, 4096x4096, w_bits 3 and 8, batch 1: unpack + gather + matmul once; matmul "
-                      "alone on the dequantised fp32 weight, mean of 5"}
+        cpu = cpu_baseline(torch, synth, shapes)
 
     if machine:
         # how much of a step is the fixed cost of its 42 dependent launches, and the rate of the rest
@@ -392,6 +430,7 @@ def main():
         "roofline": roofline, "cpu_baseline": cpu, "grouped_launches": grouped, "machine_reference": machine,
         "layers": table,
         "dequant_kbit": dequant_table, "batch_us": batch_table,
+        "llama3_8b_batches": llama3, "dequant_layer_set": dequant_layer,
     }
     if args.table and table:
         with open(args.table, "w") as f:
@@ -411,6 +450,86 @@ def main():
                 for r in batch_table:
                     f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | " + " | ".join(f"{r[f'us_M{M}']:.1f}" for M in batches) + " |\n")
     print(json.dumps(result))
+
+
+def _cpu_model() -> str:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(torch, synth, shapes):
+    """Two CPU legs, about 10 s together.  (1) `value`: the C oracle's host-speed GEMV (unpack + gather + fp32
+    dot, OpenMP over rows) on two shapes x two bit-widths.  (2) `torch_reference_semantics`: the reference's
+    semantics written with PyTorch CPU ops on 4096 x 4096 at batch 1 -- bitplane unpack (shifts and masks on
+    the int32 tensor), table gather (any_precision/evaluate/eval.py:104-105), fp32 matmul
+    (any_precision/modules/AnyPrecisionLinear.py:60-62) -- for every w_bits 3..8: one warm-up, five timed
+    runs, median; end to end and the matmul alone on the dequantised weight."""
+    import numpy as np
+    import oracle
+    oracle.build()
+    rng = np.random.default_rng(0)
+    t_cpu, b_cpu = 0.0, 0
+    for _, N, K in [shapes[0], shapes[4]]:
+        qw = rng.integers(-2**31, 2**31 - 1, size=(8, N, K // 32), dtype=np.int64).astype(np.int32)
+        x = rng.normal(0, 1, size=(1, K)).astype(np.float16)
+        for b in (3, 8):
+            lut = np.sort(rng.normal(0, 0.02, size=(N, 1 << b)), axis=1).astype(np.float16)
+            oracle.matmul_kbit_fast(x, qw, lut, b)                  # warm
+            reps, t0 = 0, time.perf_counter()
+            while reps < 3 or time.perf_counter() - t0 < 1.0:       # about 1 s per case
+                oracle.matmul_kbit_fast(x, qw, lut, b)
+                reps += 1
+            t_cpu += (time.perf_counter() - t0) / reps
+            b_cpu += synth.gemv_bytes(N, K, b, 1)
+    cpu = {"value": round(b_cpu / t_cpu / 1e9, 3), "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+           "sample": "C oracle GEMV (unpack+gather+fp32 dot, OpenMP over rows): 4096x4096 and 11008x4096 at w_bits "
+                     "3 and 8, batch 1, each repeated for about 1 s (mean)"}
+
+    N = K = 4096
+    torch.set_num_threads(os.cpu_count() or 1)
+    qw_t = torch.from_numpy(rng.integers(-2**31, 2**31 - 1, size=(8, N, K // 32), dtype=np.int64).astype(np.int32))
+    x_t = torch.from_numpy(rng.normal(0, 1, size=(1, K)).astype(np.float32))
+    shifts = torch.arange(7, -1, -1, dtype=torch.uint8)
+
+    def torch_unpack(b):
+        by = qw_t[:b].contiguous().view(torch.uint8).view(b, N, K // 1024, 32, 4).flip(-1)        # [p,n,c,t,j]
+        bits = (by.unsqueeze(-1) >> shifts) & 1                                                   # [p,n,c,t,j,e]
+        bits = bits.permute(0, 1, 2, 4, 3, 5).reshape(b, N, K)
+        w = (1 << torch.arange(b - 1, -1, -1, dtype=torch.int64)).view(b, 1, 1)
+        return (bits.to(torch.int64) * w).sum(0)
+
+    per_bits = []
+    for b in BITS:
+        lut_t = torch.from_numpy(np.sort(rng.normal(0, 0.02, size=(N, 1 << b)), axis=1).astype(np.float32))
+        e2e, mm = [], []
+        for rep in range(6):                                        # the first run is the warm-up
+            t0 = time.perf_counter()
+            wdq = torch.gather(lut_t, 1, torch_unpack(b))
+            y = x_t @ wdq.T
+            t1 = time.perf_counter()
+            y = x_t @ wdq.T
+            t2 = time.perf_counter()
+            if rep:
+                e2e.append(t1 - t0)
+                mm.append(t2 - t1)
+        e2e.sort()
+        mm.sort()
+        by_b = synth.gemv_bytes(N, K, b, 1)
+        per_bits.append({"w_bits": b, "ms_end_to_end": round(e2e[len(e2e) // 2] * 1e3, 2),
+                         "ms_matmul_only": round(mm[len(mm) // 2] * 1e3, 3),
+                         "GBps_end_to_end": round(by_b / e2e[len(e2e) // 2] / 1e9, 4)})
+    cpu["torch_reference_semantics"] = {
+        "per_w_bits": per_bits, "os_cpu_count": os.cpu_count(), "torch_threads": torch.get_num_threads(),
+        "cpu_model": _cpu_model(),
+        "sample": "torch CPU ops, 4096x4096, batch 1, every w_bits 3..8: unpack + gather + fp32 matmul end to end, "
+                  "and the matmul alone on the dequantised fp32 weight; one warm-up, median of five"}
+    return cpu
 
 
 def _graph_us(torch, side, enqueue, reps):

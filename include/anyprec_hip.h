@@ -92,6 +92,18 @@ int ap_abi_version(void);
 int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits,
                             int *wpl, int *segments, int *rows, int *grid);
 
+/* Which kernel ap_matmul_kbit would launch for one linear (output taken to be 4-byte aligned), for
+ * reports and tests.  Returns AP_OK or the argument errors of ap_matmul_kbit. */
+enum {
+    AP_ROUTE_DOT = 0,     /* gemv_kbit_kernel: one or two rows per workgroup, one word per lane         */
+    AP_ROUTE_STREAM = 1,  /* gemvp_kbit_kernel: row pairs, 16-byte plane loads, few long waves           */
+    AP_ROUTE_FINE = 2,    /* gemvf_kbit_kernel: one workgroup per row pair, 8-byte plane loads           */
+    AP_ROUTE_PERSIST = 3, /* gemvr_kbit_kernel: persistent row loop (only when forced)                   */
+    AP_ROUTE_MFMA4 = 4,   /* gemv4_kbit_kernel: 4x4x4 matrix-core kernel                                 */
+    AP_ROUTE_MFMA16 = 5   /* gemm_kbit_kernel: 16x16x32 matrix-core kernel                               */
+};
+int ap_matmul_kbit_route(int M, int N, int K, int w_bits, int *route);
+
 /* Test and measurement hook, no counterpart in the reference: overrides one launch-heuristic knob
  * (which kernel variant serves a shape, grid sizes) for the whole process, so that tests can force
  * every variant onto shapes they can check and benchmarks can sweep.  Results never depend on a knob

@@ -93,3 +93,25 @@ def test_tuning_knobs_need_no_gpu():
     with _capi.tuning(gemv_rows=2):
         assert _capi.matmul_geometry(1, 4096, 4096, 4)["rows"] == 2
     assert _capi.matmul_geometry(1, 4096, 4096, 4)["rows"] == 1
+
+
+def test_route_report_follows_the_rule_and_the_knobs():
+    """ap_matmul_kbit_route names the kernel a single linear gets; forcing knobs change it at once."""
+    from any_precision_amd import _capi
+    assert _capi.matmul_route(1, 4096, 4096, 4) == "dot"
+    assert _capi.matmul_route(1, 11008, 4096, 3) == "stream"
+    assert _capi.matmul_route(1, 11008, 4096, 8) == "fine"
+    assert _capi.matmul_route(1, 4096, 11008, 3) == "dot"
+    assert _capi.matmul_route(2, 4096, 14336, 4) == "stream"
+    assert _capi.matmul_route(8, 4096, 4096, 4) == "mfma16"
+    assert _capi.matmul_route(8, 14336, 4096, 4) == "mfma4"
+    assert _capi.matmul_route(1, 8, 32 * 64 * 2 * 17, 4) == "mfma16"      # longer than a workgroup covers
+    with _capi.tuning(gemv_stream=0, gemv_fine=0):
+        assert _capi.matmul_route(1, 11008, 4096, 3) == "dot"
+    with _capi.tuning(gemv_persist=2):
+        assert _capi.matmul_route(3, 64, 4096, 5) == "persist"
+        assert _capi.matmul_route(3, 64, 4128, 5) != "persist"            # rows must be a multiple of 64 elements
+    with _capi.tuning(gemv_fine=2):
+        assert _capi.matmul_route(1, 63, 4096, 5) == "dot"                # odd row count: not served
+    with pytest.raises(ValueError):
+        _capi.matmul_route(9, 64, 4096, 5)
