@@ -41,6 +41,8 @@ lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi]
 lib.ap_matmul_kbit_geometry.restype = _ci
 lib.ap_probe_stream.argtypes = [_vp, ctypes.c_longlong, _vp, ctypes.c_longlong, _vp, _ci, _vp]
 lib.ap_probe_stream.restype = _ci
+lib.ap_probe_write.argtypes = [_vp, ctypes.c_longlong, ctypes.c_uint32, _ci, _vp]
+lib.ap_probe_write.restype = _ci
 lib.ap_probe_empty.argtypes = [_vp, _vp]
 lib.ap_probe_empty.restype = _ci
 lib.ap_matmul_kbit_route.argtypes = [_ci, _ci, _ci, _ci, _pi]
@@ -56,7 +58,7 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
     )
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
-           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_matmul_kbit_route")
+           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_probe_write", "ap_matmul_kbit_route")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
 

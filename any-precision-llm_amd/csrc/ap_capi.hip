@@ -192,6 +192,22 @@ int ap_probe_stream(const void *buf0, long long bytes0, const void *buf1, long l
     return launch_status();
 }
 
+int ap_probe_write(void *dst, long long bytes, uint32_t value, int waves_per_cu, void *stream) {
+    if (!dst) return AP_ENULL;
+    if (bytes < 0 || (bytes & 15)) return AP_ESHAPE;
+    if (!aligned16(dst)) return AP_EALIGN;
+    if (waves_per_cu < 1) waves_per_cu = 32;
+    const long long units = bytes >> 4;
+    long long blocks = (long long)cu_count() * waves_per_cu / kProbeWaves;
+    const long long need = (units + kProbeWaves * kWave - 1) / (kProbeWaves * kWave);
+    if (blocks > need) blocks = need;
+    if (blocks < 1) blocks = 1;
+    drain_stale_error();
+    probe_write_kernel<<<dim3((unsigned)blocks), dim3(kProbeWaves * kWave), 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<u32x4 *>(dst), units, value);
+    return launch_status();
+}
+
 int ap_probe_empty(uint32_t *sink, void *stream) {
     if (!sink) return AP_ENULL;
     drain_stale_error();

@@ -33,6 +33,16 @@ __global__ __launch_bounds__(kProbeWaves *kWave) void probe_stream_kernel(const 
     if (v == 0x9e3779b9u) sink[0] = v;  // practically never true: no store traffic, loads stay live
 }
 
+// Only WRITES `units` 16-byte units (non-temporal stores of a constant): what the machine does for the
+// output of a kernel that is bound by its stores, such as the dequantiser.
+__global__ __launch_bounds__(kProbeWaves *kWave) void probe_write_kernel(u32x4 *__restrict__ dst, long long units,
+                                                                          uint32_t value) {
+    const long long tid = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    const u32x4 v = {value, value, value, value};
+    for (long long i = tid; i < units; i += stride) __builtin_nontemporal_store(v, dst + i);
+}
+
 // A kernel that does nothing: the fixed cost of a launch.
 __global__ void probe_empty_kernel(uint32_t *sink) {
     if (threadIdx.x == 0x7fffffffu) sink[0] = 0u;  // never true: the kernel keeps its argument and stores nothing

@@ -291,11 +291,22 @@ def main():
                 if rc != 0:
                     raise RuntimeError(_capi.strerror(rc))
 
+            def write_only(st):
+                state["i"] = (state["i"] + 1) % nout
+                rc = lib.ap_probe_write(outs[state["i"]].data_ptr(), 2 * N * K, 7, 32, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+
+            # a kernel that only WRITES the fp16 output (no planes, no lookups): the store floor of this box
+            us_write = time_graph(write_only, 12)
             for b in BITS:
                 us = time_graph(lambda st: deq(st, b), 12)
                 by = synth.dequant_bytes(N, K, b)
+                us_read = next((r["stream_only_us"] for r in table if (r["N"], r["K"], r["w_bits"]) == (N, K, b)), None)
                 dequant_table.append({"N": N, "K": K, "w_bits": b, "us": round(us, 2),
-                                      "GBps": round(by / us / 1e3, 1), "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4)})
+                                      "GBps": round(by / us / 1e3, 1), "frac": round(by / us / 1e3 / HBM_PEAK_GBS, 4),
+                                      "write_only_us": round(us_write, 2), "read_only_us": us_read,
+                                      "frac_of_write_floor": round(us_write / us, 4)})
             del outs
         # batches: matmul_kbit for M <= 8 (MFMA kernel from 5 rows on), fused gemm_kbit for 16 and 32 rows
         for (N, K) in pools:

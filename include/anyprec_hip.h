@@ -118,9 +118,12 @@ int ap_get_tuning(const char *name, int *value);
  * and bytes1 bytes at buf1 (multiples of 16; buf1 may be NULL with bytes1 = 0) with 16-byte non-temporal
  * loads from `waves_per_cu` waves per CU (<= 0: 8) and writes nothing but possibly sink[0]: timed over
  * the planes and tables of a linear it is the floor any kernel over those bytes has on this machine.
+ * ap_probe_write only WRITES `bytes` bytes (a multiple of 16) of `value` at dst with 16-byte non-temporal
+ * stores (waves_per_cu <= 0: 32): the floor of a store-bound kernel such as ap_dequant_kbit.
  * ap_probe_empty launches one wave that does nothing: the fixed cost of a launch. */
 int ap_probe_stream(const void *buf0, long long bytes0, const void *buf1, long long bytes1,
                     uint32_t *sink, int waves_per_cu, void *stream);
+int ap_probe_write(void *dst, long long bytes, uint32_t value, int waves_per_cu, void *stream);
 int ap_probe_empty(uint32_t *sink, void *stream);
 
 #ifdef __cplusplus
