@@ -34,18 +34,17 @@ LLAMA_ARCH_CONFIG = {
 }
 
 
-def replace_module_by_name(layer, module_name, new_module):
-    levels = module_name.split(".")
-    module = layer
-    for level in levels[:-1]:
-        module = getattr(module, level) if not level.isdigit() else module[int(level)]
-    setattr(module, levels[-1], new_module)
-
-
 def _get_by_name(root, dotted):
-    for name in dotted.split("."):
-        root = getattr(root, name)
+    """Sub-module ``a.b.0.c`` of ``root`` (numeric parts index into module lists)."""
+    for part in dotted.split("."):
+        root = root[int(part)] if part.isdigit() else getattr(root, part)
     return root
+
+
+def _set_by_name(root, dotted, module):
+    """Puts ``module`` where ``dotted`` names a sub-module of ``root``."""
+    parent, _, leaf = dotted.rpartition(".")
+    setattr(_get_by_name(root, parent) if parent else root, leaf, module)
 
 
 class AnyPrecisionForCausalLM(nn.Module):
@@ -155,7 +154,7 @@ class AnyPrecisionForCausalLM(nn.Module):
                                         bias=module.bias is not None, precisions=self.precisions,
                                         device=module.weight.device, dtype=torch.float16)
                 self.ap_linears.append(ap)
-                replace_module_by_name(layer, name, ap)
+                _set_by_name(layer, name, ap)
 
     def _load_checkpoint(self, model_path):
         path = os.path.join(model_path, "pytorch_model.bin")
@@ -170,6 +169,10 @@ class AnyPrecisionForCausalLM(nn.Module):
 
     def save_quantized(self, output_model_path):
         """Writes the directory the reference packer writes (pack.py:165-177), minus the tokenizer."""
+        if set(self.precisions) != set(self.supported_bits):
+            # prune_precisions() has dropped planes and tables that config.anyprec still promises
+            raise RuntimeError(f"this model was loaded with precisions {self.precisions} of {self.supported_bits} and "
+                               "holds only their planes and tables: load it with every precision to save it")
         os.makedirs(output_model_path, exist_ok=True)
         state = {k: v.detach().cpu() for k, v in self.model.state_dict().items()}
         torch.save(state, os.path.join(output_model_path, "pytorch_model.bin"))

@@ -37,7 +37,8 @@ def forward_group(modules, x, precision=None, concat=False):
     stub, AnyPrecisionForCausalLM.py:168-172)."""
     rows = x.numel() // x.shape[-1]
     w_bits = modules[0].precision if precision is None else precision
-    if rows > 4 or not 2 <= len(modules) <= 4 or not x.is_contiguous() or any(
+    x = x.contiguous()
+    if rows > 4 or not 2 <= len(modules) <= 4 or any(
             m.in_features != modules[0].in_features for m in modules):
         outs = [m(x, precision=w_bits) for m in modules]
         return torch.cat(outs, dim=-1) if concat else outs
@@ -103,9 +104,10 @@ class AnyPrecisionLinear(nn.Module):
         table = self._buffers[f"lut{w_bits}"]
         rows = x.numel() // x.shape[-1]
         if rows <= 8:                                       # GEMV / skinny kernels (reference: :63-64)
-            y = matmul_kbit(x, self.qweight, table, w_bits)
-        elif fused_gemm_pays(rows, self.out_features, w_bits) and x.is_contiguous():
-            y = gemm_kbit(x, self.qweight, table, w_bits)   # fused dequant -> MFMA, weight never materialised
+            # the ops take dense row-major activations; a transposed or sliced view is copied (a no-op otherwise)
+            y = matmul_kbit(x.contiguous(), self.qweight, table, w_bits)
+        elif fused_gemm_pays(rows, self.out_features, w_bits):
+            y = gemm_kbit(x.contiguous(), self.qweight, table, w_bits)   # fused dequant -> MFMA, weight never materialised
         else:                                               # reference: :60-62
             y = torch.matmul(x, dequant_kbit(self.qweight, table, w_bits).T)
         if self.bias is not None:

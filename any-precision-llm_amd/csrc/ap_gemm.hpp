@@ -275,6 +275,10 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
                 } else {
                     afrag = a[t][mb];
                 }
+                // words past the row end: zero activations as well as zero weights (0 * inf would be NaN)
+                if constexpr (CHECK) {
+                    if (!live[wi]) afrag = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                }
 #pragma unroll
                 for (int rb = 0; rb < RB; rb++)
                     acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag[rb], acc[rb][mb], 0, 0, 0);

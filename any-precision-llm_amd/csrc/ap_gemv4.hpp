@@ -159,7 +159,9 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
                 }
                 const uint32_t lo = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a0);
                 const uint32_t hi = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a1);
-                bw[i] = lo | (hi << 16);
+                // words past the row end: zero weights as well as zero activations, so that a non-finite
+                // table entry or activation there cannot turn 0 * inf into NaN
+                bw[i] = live[g] ? (lo | (hi << 16)) : 0u;
             });
 #pragma unroll
             for (int h = 0; h < 2; h++) {

@@ -44,6 +44,22 @@ def test_forward_every_branch_and_bias(oracle):
             assert_close_gemv(y, want + bias, f"b={b} M={M}")
 
 
+def test_strided_activations_are_accepted_on_every_branch(oracle):
+    """A transposed or sliced activation view (as Hugging Face modules hand over now and then) gives the
+    result of its dense copy on the GEMV, the fused-GEMM and the dequant + matmul branch alike."""
+    L = make(96, 2048, seed=4)
+    m, sd = _module(L, bias=False)
+    for M in (1, 4, 8, 20, 70):
+        x = synth.make_x(M, 2 * L.K, seed=M)
+        xg = torch.from_numpy(x).cuda()[:, ::2]                 # every other column: stride 2
+        assert not xg.is_contiguous()
+        _, want = oracle.matmul_kbit(np.ascontiguousarray(x[:, ::2]), L.qweight, L.luts[4], 4, return_f64=True)
+        assert_close_gemv(m(xg, precision=4), want, f"strided M={M}")
+        xt = torch.from_numpy(np.ascontiguousarray(x[:, ::2].T)).cuda().T    # transposed view of a [K, M] tensor
+        assert not xt.is_contiguous() or M == 1
+        assert_close_gemv(m(xt, precision=4), want, f"transposed M={M}")
+
+
 def test_set_precision_and_prune(oracle):
     L = make(32, 1024, seed=2)
     m, _ = _module(L, bias=False, precisions=[3, 4, 6])

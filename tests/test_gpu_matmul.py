@@ -311,3 +311,33 @@ def test_denormal_table_entries_are_not_flushed(ext, oracle):
             _, want = oracle.matmul_kbit(x, L.qweight, lut, b, return_f64=True)
             assert np.abs(want).max() > 5e-6
             assert_close_gemv(got, want, f"denormal tables b={b} M={M}")
+
+
+def test_non_finite_values_stay_where_they_belong(ext):
+    """An infinite table entry makes exactly the outputs of its row infinite, an infinite activation
+    exactly the outputs of its activation row -- also on rows whose last step reaches past the row end
+    (K = 11008: 344 words, not a multiple of what a step of the matrix-core kernels covers), where words
+    past the end must contribute zeros and not 0 * inf.  Reference: fp32 matmul of the dequantised weight."""
+    N, K = 48, 11008
+    L = make(N, K, seed=9)
+    q, luts = layer_to_gpu(L)
+    for b in (3, 8):
+        lut = luts[b].clone()
+        lut[5, :] = float("inf")                           # every entry of row 5
+        w = ext.dequant_kbit(q, lut, b)
+        for M in (1, 2, 4, 8):
+            x = torch.from_numpy(synth.make_x(M, K, seed=M)).cuda().abs() + 0.01      # positive: inf rows give +inf, not NaN
+            for fn in (ext.matmul_kbit, ext.gemm_kbit):
+                print(f"non-finite b={b} M={M} {fn.__name__}", flush=True)
+                y = fn(x, q, lut, b)
+                assert torch.isinf(y[:, 5]).all() and (y[:, 5] > 0).all()
+                rest = torch.cat([y[:, :5], y[:, 6:]], dim=1)
+                assert torch.isfinite(rest).all()
+                want = (x.double() @ w.double().T)
+                want = torch.cat([want[:, :5], want[:, 6:]], dim=1)
+                assert (rest.double() - want).norm() <= 1e-2 * want.norm()
+            if M >= 2:
+                x2 = x.clone()
+                x2[1, -1] = float("inf")                   # last element of activation row 1
+                y = ext.matmul_kbit(x2, q, luts[b], b)
+                assert torch.isfinite(y[0]).all() and not torch.isfinite(y[1]).any()

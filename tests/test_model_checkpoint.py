@@ -68,6 +68,11 @@ def test_checkpoint_directory_round_trip(model, tmp_path):
     lin = pruned.ap_linears[0]
     assert lin.qweight.shape[0] == 5 and hasattr(lin, "lut3") and not hasattr(lin, "lut8")
     assert torch.equal(lin.qweight, model.ap_linears[0].qweight[:5])
+    # a model that holds a subset of the precisions has dropped planes and tables the config still promises:
+    # saving it would write a checkpoint that cannot be loaded again
+    with pytest.raises(RuntimeError, match="every precision"):
+        pruned.save_quantized(str(tmp_path / "pruned"))
+    assert not os.path.exists(tmp_path / "pruned")
 
 
 def test_rejects_foreign_checkpoints(tmp_path):
