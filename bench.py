@@ -34,14 +34,17 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--workload", default="llama2_7b_layer_batch1",
                     choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model",
-                             "llama2_7b_decode", "llama2_7b_prefill"),
+                             "llama2_7b_decode", "llama2_7b_prefill", "gemv_kernel_variants"),
                     help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
                          "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
                          "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.  "
                          "llama2_7b_decode: batch-1 greedy decoding of a random-init Llama-2-7B-shaped model, "
                          "256 tokens after a 128-token prompt, per w_bits.  "
                          "llama2_7b_prefill: the seven linears of a layer on 32 x 512 = 16384 activation rows "
-                         "(dequant_kbit + library GEMM, the large-batch branch of AnyPrecisionLinear).")
+                         "(dequant_kbit + library GEMM, the large-batch branch of AnyPrecisionLinear).  "
+                         "gemv_kernel_variants: the four dot-product GEMV kernels forced in turn (tuning knobs) on "
+                         "the headline shapes and on 28672 x 8192, batch 1, beside the read-only stream; with "
+                         "--eager the launches go out one by one (the form rocprofv3 counter runs need).")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -95,6 +98,8 @@ def main():
         return dequant_full_model(args, torch, _capi, synth)
     if args.workload == "llama2_7b_prefill":
         return prefill_linears(args, torch, _capi, synth)
+    if args.workload == "gemv_kernel_variants":
+        return gemv_kernel_variants(args, torch, _capi, synth)
     if args.workload == "llama2_7b_decode":
         with torch.inference_mode():     # the decoder captures its graphs in inference mode; stay in it
             return decode_tokens(args, torch, _capi, synth)
@@ -613,6 +618,79 @@ def batch_sweep(args, torch, _capi, synth):
                                "down 4096x14336), M in 1,2,4,8, parent 8 bits, w_bits 3..8; per-kernel graphs of "
                                f"{args.kernel_reps} launches over cold weight sets"},
         "kernels": rows}))
+
+
+def gemv_kernel_variants(args, torch, _capi, synth):
+    """Batch-1 GEMV with each of the four dot-product kernels forced in turn, cold weight sets: us per launch
+    and fraction of the HBM peak per (shape, w_bits, kernel), beside a kernel that only reads the same bytes.
+    With --eager nothing is timed in a graph: every launch goes out on its own (kernel names and counters
+    of a rocprofv3 run then belong to single launches); the printed times then include host launch cost."""
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    side = torch.cuda.Stream()
+    sink = torch.zeros(16, dtype=torch.int32, device="cuda")
+    variants = (("dot", {}), ("fine", {"gemv_fine": 2}), ("stream", {"gemv_stream": 2}), ("persist", {"gemv_persist": 2}))
+    off = {"gemv_fine": 0, "gemv_stream": 0, "gemv_persist": 0}
+    bits = (3, 5, 8)
+    rows = []
+    for N, K in ((4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192)):
+        sets = max(3, int(args.pool_gb * 1e9 / (3 * N * K / 8)) + 1)
+        if args.eager:
+            sets = min(sets, 12)
+        P = WeightPool(torch, N, K, sets, gen, bits=bits)
+        x = torch.randn((1, K), device="cuda", generator=gen).to(torch.float16)
+        cur = {"j": 0}
+        for b in bits:
+            by = synth.gemv_bytes(N, K, b, 1)
+            reps = min(P.sets, max(8, int(1e9 / by) + 1))
+
+            def read_only(st):
+                cur["j"] = (cur["j"] + 1) % P.sets
+                rc = lib.ap_probe_stream(P.qweight[cur["j"]].data_ptr(), b * N * K // 8, P.luts[b][cur["j"]].data_ptr(),
+                                         N * (2 << b), sink.data_ptr(), 32, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+
+            def gemv(st):
+                cur["j"] = (cur["j"] + 1) % P.sets
+                rc = lib.ap_matmul_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                        P.out.data_ptr(), 1, N, K, b, st)
+                if rc != 0:
+                    raise RuntimeError(_capi.strerror(rc))
+
+            def timed(fn):
+                if not args.eager:
+                    return _graph_us(torch, side, fn, reps)
+                with torch.cuda.stream(side):
+                    fn(side.cuda_stream)
+                    side.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(reps):
+                        fn(side.cuda_stream)
+                    side.synchronize()
+                return (time.perf_counter() - t0) * 1e6 / reps
+
+            row = {"N": N, "K": K, "w_bits": b, "bytes": by, "stream_only_us": round(timed(read_only), 2)}
+            for name, knobs in variants:
+                with _capi.tuning(**{**off, **knobs}):
+                    if _capi.matmul_route(1, N, K, b) != name:
+                        continue
+                    us = timed(gemv)
+                row[f"{name}_us"] = round(us, 2)
+                row[f"{name}_frac"] = round(by / us / 1e3 / HBM_PEAK_GBS, 4)
+            row["default_kernel"] = _capi.matmul_route(1, N, K, b)
+            rows.append(row)
+        del P
+        torch.cuda.empty_cache()
+    print(json.dumps({
+        "metric": "bitplane GEMV us per launch by kernel variant, batch 1", "unit": "us", "n_gpus": 1,
+        "higher_is_better": False, "vs_baseline": None, "data": "synthetic",
+        "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate",
+        "config": {"workload": "4096x4096, 11008x4096, 4096x11008, 28672x8192 at w_bits 3, 5, 8, batch 1; each of the "
+                               "dot / fine / stream / persist kernels forced through ap_set_tuning; cold weight sets; "
+                               + ("eager launches" if args.eager else "HIP graphs")},
+        "value": None, "kernels": rows}))
 
 
 def dequant_full_model(args, torch, _capi, synth):
