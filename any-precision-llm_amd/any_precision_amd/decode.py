@@ -6,9 +6,11 @@ Hugging Face loop (demo.py:59-80), which at batch 1 is bound by Python and launc
 not by the kernels.  Here one decode step -- embedding, 32 x (norm, q/k/v GEMV, rotary,
 cache write, attention over a static cache, o GEMV, norm, gate/up GEMV, SiLU, down GEMV),
 final norm, head, argmax, position increment -- is recorded once per precision and replayed
-per token: no host work between tokens, 19 kernel launches per layer.  Only the seven linears per layer are this
-library's kernels (q/k/v and gate/up as one grouped launch each); everything else is stock
-PyTorch ops, as in the reference.
+per token: no host work between tokens.  With ``fused_ops`` (the default) a layer is 9 launches, all
+of this library: the seven linears (q/k/v and gate/up as one grouped launch each), residual add +
+RMSNorm twice, rotary + cache append + attention in one kernel, SiLU * up.  Without it everything
+but the linears is stock PyTorch ops, as in the reference (19 launches per layer); that path also
+serves the prompt and is what the fused one is tested against.
 
 Supports Llama-style decoders (RMSNorm, rotary attention with optional grouped KV heads,
 SwiGLU MLP, no biases in norms); anything else raises.
@@ -20,6 +22,7 @@ import math
 import torch
 import torch.nn.functional as F
 
+from . import _capi
 from .linear import forward_group
 
 
@@ -30,8 +33,10 @@ def _rope(x, cos, sin_signed):
 
 
 class GraphDecoder:
-    def __init__(self, ap_model, max_len=512, group_launches=True):
-        """``group_launches``: issue the q/k/v and the gate/up GEMVs of a layer as one launch each."""
+    def __init__(self, ap_model, max_len=512, group_launches=True, fused_ops=True):
+        """``group_launches``: issue the q/k/v and the gate/up GEMVs of a layer as one launch each.
+        ``fused_ops``: the decode step runs the library's add + RMSNorm, attention and SiLU * up kernels
+        instead of stock PyTorch ops (head sizes 32, 64, 128, 256 and caches of up to 8192 rows)."""
         self.group_launches = group_launches
         cfg = ap_model.config
         if getattr(cfg, "model_type", None) != "llama":
@@ -80,6 +85,17 @@ class GraphDecoder:
         self.logits = torch.zeros((1, self.head.shape[0]), dtype=torch.float16, device=dev)
         self.graphs = {}
         self.stream = torch.cuda.Stream(device=dev)
+        self.fused_ops = bool(fused_ops) and self.hd in (32, 64, 128, 256) and max_len <= 8192
+        if self.fused_ops:
+            # fp32 rotary tables [max_len, hd / 2] and the static buffers of the fused step
+            self.cos32 = ang[:, :self.hd // 2].cos().contiguous()
+            self.sin32 = ang[:, :self.hd // 2].sin().contiguous()
+            H, I = cfg.hidden_size, cfg.intermediate_size
+            f16 = dict(dtype=torch.float16, device=dev)
+            self.f_h = torch.zeros((1, H), **f16)        # residual stream
+            self.f_x = torch.zeros((1, H), **f16)        # normalised input of the next linears
+            self.f_ctx = torch.zeros((1, self.nh * self.hd), **f16)
+            self.f_act = torch.zeros((1, I), **f16)
 
     # ------------------------------------------------------------------ the network
     def _norm(self, x, w):
@@ -132,9 +148,45 @@ class GraphDecoder:
         h = self._norm(h[-1:], self.final_norm)
         return F.linear(h, self.head)
 
+    def _forward_fused(self, precision):
+        """The token self.tok at cache row self.pos through the network -> logits [1, vocab]; 9 launches per layer."""
+        lib, st = _capi.lib, torch.cuda.current_stream(self.dev).cuda_stream
+        H, eps = self.cfg.hidden_size, float(self.eps)
+        scale = 1.0 / math.sqrt(self.hd)
+
+        def add_norm(delta, weight):          # f_h += delta; f_x = rmsnorm(f_h) * weight
+            _capi.check(lib.ap_add_rmsnorm(self.f_h.data_ptr(), 0 if delta is None else delta.data_ptr(), weight.data_ptr(),
+                                           self.f_h.data_ptr(), self.f_x.data_ptr(), 1, H, eps, st), "ap_add_rmsnorm")
+
+        self.f_h.copy_(self.embed.index_select(0, self.tok))
+        delta = None
+        for li, layer in enumerate(self.layers):
+            att = layer.self_attn
+            add_norm(delta, layer.input_layernorm.weight)
+            if self.group_launches:
+                qkv = forward_group((att.q_proj, att.k_proj, att.v_proj), self.f_x, precision, concat=True)
+            else:
+                qkv = torch.cat([m(self.f_x, precision=precision) for m in (att.q_proj, att.k_proj, att.v_proj)], dim=-1)
+            _capi.check(lib.ap_decode_attention(qkv.data_ptr(), self.cos32.data_ptr(), self.sin32.data_ptr(),
+                                                self.kcache[li].data_ptr(), self.vcache[li].data_ptr(), self.pos.data_ptr(),
+                                                self.f_ctx.data_ptr(), self.nh, self.nkv, self.hd, self.max_len, scale, st),
+                        "ap_decode_attention")
+            add_norm(att.o_proj(self.f_ctx, precision=precision), layer.post_attention_layernorm.weight)
+            if self.group_launches:
+                gate, up = forward_group((layer.mlp.gate_proj, layer.mlp.up_proj), self.f_x, precision)
+            else:
+                gate, up = layer.mlp.gate_proj(self.f_x, precision=precision), layer.mlp.up_proj(self.f_x, precision=precision)
+            _capi.check(lib.ap_silu_mul(gate.data_ptr(), up.data_ptr(), self.f_act.data_ptr(), gate.numel(), st), "ap_silu_mul")
+            delta = layer.mlp.down_proj(self.f_act, precision=precision)
+        add_norm(delta, self.final_norm)
+        return F.linear(self.f_x, self.head)
+
     def _step(self, precision):
         """One decode step on the static state: consumes self.tok at self.pos, leaves the next token."""
-        logits = self._forward(self.tok, self.pos, precision)
+        if self.fused_ops:
+            logits = self._forward_fused(precision)
+        else:
+            logits = self._forward(self.tok, self.pos, precision)
         self.logits.copy_(logits)
         nxt = torch.argmax(logits, dim=-1)
         self.pos.add_(1)

@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include "anyprec_hip.h"
+#include "ap_decode.hpp"
 #include "ap_dequant.hpp"
 #include "ap_gemm_launch.hpp"
 #include "ap_gemv4_launch.hpp"
@@ -212,6 +213,52 @@ int ap_probe_empty(uint32_t *sink, void *stream) {
     if (!sink) return AP_ENULL;
     drain_stale_error();
     probe_empty_kernel<<<dim3(1), dim3(kWave), 0, static_cast<hipStream_t>(stream)>>>(sink);
+    return launch_status();
+}
+
+int ap_add_rmsnorm(const uint16_t *h, const uint16_t *delta, const uint16_t *weight, uint16_t *h_out, uint16_t *x_out,
+                   int rows, int H, float eps, void *stream) {
+    if (!h || !weight || !h_out || !x_out) return AP_ENULL;
+    if (rows < 1 || H < 8 || (H & 7)) return AP_ESHAPE;
+    if (!aligned16(h) || !aligned16(weight) || !aligned16(h_out) || !aligned16(x_out) || (delta && !aligned16(delta)))
+        return AP_EALIGN;
+    drain_stale_error();
+    add_rmsnorm_kernel<<<dim3(rows), dim3(kNormThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        reinterpret_cast<const half_t *>(h), reinterpret_cast<const half_t *>(delta), reinterpret_cast<const half_t *>(weight),
+        reinterpret_cast<half_t *>(h_out), reinterpret_cast<half_t *>(x_out), H, eps);
+    return launch_status();
+}
+
+int ap_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *out, long long n, void *stream) {
+    if (!gate || !up || !out) return AP_ENULL;
+    if (n < 8 || (n & 7)) return AP_ESHAPE;
+    if (!aligned16(gate) || !aligned16(up) || !aligned16(out)) return AP_EALIGN;
+    const long long blocks = (n / 8 + 255) / 256;
+    drain_stale_error();
+    silu_mul_kernel<<<dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+        reinterpret_cast<const half_t *>(gate), reinterpret_cast<const half_t *>(up), reinterpret_cast<half_t *>(out), n);
+    return launch_status();
+}
+
+int ap_decode_attention(const uint16_t *qkv, const float *cos_table, const float *sin_table, uint16_t *kcache,
+                        uint16_t *vcache, const long long *pos, uint16_t *out, int n_heads, int n_kv_heads, int head_dim,
+                        int max_len, float scale, void *stream) {
+    if (!qkv || !cos_table || !sin_table || !kcache || !vcache || !pos || !out) return AP_ENULL;
+    if (n_heads < 1 || n_kv_heads < 1 || n_heads % n_kv_heads) return AP_ESHAPE;
+    if (head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256) return AP_ESHAPE;
+    if (max_len < 1 || max_len > kAttnMaxLen) return AP_ELIMIT;
+    if (!aligned16(qkv) || !aligned16(kcache) || !aligned16(vcache) || !aligned16(out)) return AP_EALIGN;
+    const half_t *q = reinterpret_cast<const half_t *>(qkv);
+    half_t *kc = reinterpret_cast<half_t *>(kcache), *vc = reinterpret_cast<half_t *>(vcache), *o = reinterpret_cast<half_t *>(out);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid(n_heads), block(kAttnThreads);
+    drain_stale_error();
+    switch (head_dim) {
+        case 32: decode_attention_kernel<32><<<grid, block, 0, st>>>(q, cos_table, sin_table, kc, vc, pos, o, n_heads, n_kv_heads, max_len, scale); break;
+        case 64: decode_attention_kernel<64><<<grid, block, 0, st>>>(q, cos_table, sin_table, kc, vc, pos, o, n_heads, n_kv_heads, max_len, scale); break;
+        case 128: decode_attention_kernel<128><<<grid, block, 0, st>>>(q, cos_table, sin_table, kc, vc, pos, o, n_heads, n_kv_heads, max_len, scale); break;
+        default: decode_attention_kernel<256><<<grid, block, 0, st>>>(q, cos_table, sin_table, kc, vc, pos, o, n_heads, n_kv_heads, max_len, scale); break;
+    }
     return launch_status();
 }
 

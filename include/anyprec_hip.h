@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 3
+#define AP_ABI_VERSION 4
 
 enum {
     AP_OK = 0,
@@ -125,6 +125,32 @@ int ap_probe_stream(const void *buf0, long long bytes0, const void *buf1, long l
                     uint32_t *sink, int waves_per_cu, void *stream);
 int ap_probe_write(void *dst, long long bytes, uint32_t value, int waves_per_cu, void *stream);
 int ap_probe_empty(uint32_t *sink, void *stream);
+
+/* ---- The rest of a decode step, for ONE new token of a Llama-architecture decoder ----------------------
+ * The reference has no native code between its linears: its model wrapper hands the step to the Hugging
+ * Face modules (any_precision/modules/AnyPrecisionForCausalLM.py:88-97, timed by demo.py:59-80), i.e. a
+ * dozen library kernels per layer around the seven GEMVs.  These three entry points replace them in a
+ * graph-captured decode step; fp16 in memory, fp32 arithmetic, one rounding per output; 16-byte aligned
+ * pointers; nothing is allocated.
+ *
+ * ap_add_rmsnorm: for each of `rows` rows of H elements (H % 8 == 0): s = h + delta (an fp16 add; delta may
+ *   be NULL), written to h_out (may alias h); x_out = s * rsqrt(mean(s^2) + eps) * weight[H]  (LlamaRMSNorm).
+ * ap_silu_mul: out = gate / (1 + exp(-gate)) * up over n elements (n % 8 == 0)  (the SwiGLU gate).
+ * ap_decode_attention: rotary embedding, cache append and attention of the token at cache row *pos (a device
+ *   scalar, so the launch can sit in a replayed graph):
+ *     qkv   [n_heads + 2 n_kv_heads, head_dim]  query, key and value heads of the token, before the rotary embedding
+ *     cos_table, sin_table [max_len, head_dim / 2] fp32: cos / sin of (row * inverse frequency i)
+ *     kcache, vcache [n_kv_heads, max_len, head_dim]: rows 0 .. *pos-1 are read, row *pos is written
+ *     out   [n_heads * head_dim] = softmax(scale * q k^T) v per head, query head h reading key/value head
+ *           h / (n_heads / n_kv_heads); rotary convention x * cos + rotate_half(x) * sin.
+ *   head_dim 32, 64, 128 or 256; max_len <= 8192 (AP_ELIMIT beyond); a *pos outside 0 .. max_len-1 leaves every
+ *   buffer untouched.  Calls that overlap on one cache race. */
+int ap_add_rmsnorm(const uint16_t *h, const uint16_t *delta, const uint16_t *weight, uint16_t *h_out, uint16_t *x_out,
+                   int rows, int H, float eps, void *stream);
+int ap_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *out, long long n, void *stream);
+int ap_decode_attention(const uint16_t *qkv, const float *cos_table, const float *sin_table, uint16_t *kcache,
+                        uint16_t *vcache, const long long *pos, uint16_t *out, int n_heads, int n_kv_heads, int head_dim,
+                        int max_len, float scale, void *stream);
 
 #ifdef __cplusplus
 }

@@ -62,6 +62,27 @@ def test_strerror_and_argument_errors_need_no_gpu():
         _capi.check(98, "x")
 
 
+def test_decode_step_argument_errors_need_no_gpu():
+    from any_precision_amd import _capi
+    L = _capi.lib
+    fake = 4096
+    assert L.ap_add_rmsnorm(None, None, fake, fake, fake, 1, 128, 1e-5, None) == _capi.AP_ENULL
+    assert L.ap_add_rmsnorm(fake, None, fake, fake, fake, 0, 128, 1e-5, None) == _capi.AP_ESHAPE
+    assert L.ap_add_rmsnorm(fake, None, fake, fake, fake, 1, 100, 1e-5, None) == _capi.AP_ESHAPE
+    assert L.ap_add_rmsnorm(fake, fake + 2, fake, fake, fake, 1, 128, 1e-5, None) == _capi.AP_EALIGN
+    assert L.ap_silu_mul(fake, None, fake, 64, None) == _capi.AP_ENULL
+    assert L.ap_silu_mul(fake, fake, fake, 12, None) == _capi.AP_ESHAPE
+    assert L.ap_silu_mul(fake, fake, fake + 4, 64, None) == _capi.AP_EALIGN
+    att = lambda **kw: L.ap_decode_attention(*[kw.get(k, d) for k, d in (
+        ("qkv", fake), ("cos", fake), ("sin", fake), ("kc", fake), ("vc", fake), ("pos", fake), ("out", fake),
+        ("nh", 8), ("nkv", 2), ("hd", 128), ("max_len", 512), ("scale", 0.1), ("stream", None))])
+    assert att(pos=None) == _capi.AP_ENULL
+    assert att(nkv=3) == _capi.AP_ESHAPE          # query heads must be a multiple of the key/value heads
+    assert att(hd=96) == _capi.AP_ESHAPE
+    assert att(max_len=8193) == _capi.AP_ELIMIT
+    assert att(kc=fake + 8) == _capi.AP_EALIGN
+
+
 def test_geometry_covers_rows_and_words():
     from any_precision_amd import _capi
     for M in (1, 2, 4, 8):
