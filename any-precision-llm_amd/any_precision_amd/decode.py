@@ -6,8 +6,8 @@ Hugging Face loop (demo.py:59-80), which at batch 1 is bound by Python and launc
 not by the kernels.  Here one decode step -- embedding, 32 x (norm, q/k/v GEMV, rotary,
 cache write, attention over a static cache, o GEMV, norm, gate/up GEMV, SiLU, down GEMV),
 final norm, head, argmax, position increment -- is recorded once per precision and replayed
-per token: no host work between tokens.  With ``fused_ops`` (the default) a layer is 9 launches, all
-of this library: the seven linears (q/k/v and gate/up as one grouped launch each), residual add +
+per token: no host work between tokens.  With ``fused_ops`` (the default) a layer is 8 launches, all
+of this library: the seven linears in four (q/k/v and gate/up as one grouped launch each), residual add +
 RMSNorm twice, rotary + cache append + attention in one kernel, SiLU * up.  Without it everything
 but the linears is stock PyTorch ops, as in the reference (19 launches per layer); that path also
 serves the prompt and is what the fused one is tested against.
@@ -149,7 +149,7 @@ class GraphDecoder:
         return F.linear(h, self.head)
 
     def _forward_fused(self, precision):
-        """The token self.tok at cache row self.pos through the network -> logits [1, vocab]; 9 launches per layer."""
+        """The token self.tok at cache row self.pos through the network -> logits [1, vocab]; 8 launches per layer."""
         lib, st = _capi.lib, torch.cuda.current_stream(self.dev).cuda_stream
         H, eps = self.cfg.hidden_size, float(self.eps)
         scale = 1.0 / math.sqrt(self.hd)

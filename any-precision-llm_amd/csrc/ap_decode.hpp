@@ -14,7 +14,7 @@ namespace ap {
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 
 constexpr int kNormThreads = 256;
-constexpr int kAttnThreads = 512;  // eight waves: the kernel is a chain of load latencies, more waves = more loads in flight
+constexpr int kAttnThreads = 1024;  // sixteen waves: the kernel is a chain of load latencies, more waves = more loads in flight
 constexpr int kAttnMaxLen = 8192;  // cache rows one launch can attend over (scores live in LDS)
 
 __device__ __forceinline__ float wave_max(float v) {

@@ -427,6 +427,14 @@ def main():
     if not args.no_cpu:
         cpu = cpu_baseline(torch, synth, shapes)
 
+    # ---- the model-level figure of the same path: batch-1 decode of the Llama-2-7B-shaped model (3 and 8 bits)
+    decode = None
+    sets_per_shape = {f"{N}x{K}": P.sets for (N, K), P in pools.items()}
+    if not args.only_step and not args.no_extras and not args.eager:
+        pools.clear()               # the weight pools are no longer needed: make room for the model
+        torch.cuda.empty_cache()
+        decode = decode_summary(torch)
+
     if machine:
         # how much of a step is the fixed cost of its 42 dependent launches, and the rate of the rest
         floor_ms = len(BITS) * len(shapes) * machine["graph_node_us"] / 1e3
@@ -440,13 +448,13 @@ def main():
         "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate", "data": "synthetic",
         "config": {"workload": "Llama-2-7B decoder-layer linear set (q,k,v,o 4096x4096; gate,up 11008x4096; "
                                "down 4096x11008), batch 1, parent 8 bits, w_bits 3..8 = 42 GEMVs per step",
-                   "weight_sets_per_shape": {f"{N}x{K}": P.sets for (N, K), P in pools.items()},
+                   "weight_sets_per_shape": sets_per_shape,
                    "bytes_per_step": step_bytes,
                    "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4)},
         "roofline": roofline, "cpu_baseline": cpu, "grouped_launches": grouped, "machine_reference": machine,
         "layers": table,
         "dequant_kbit": dequant_table, "batch_us": batch_table,
-        "llama3_8b_batches": llama3, "dequant_layer_set": dequant_layer,
+        "llama3_8b_batches": llama3, "dequant_layer_set": dequant_layer, "llama2_7b_decode": decode,
     }
     if args.table and table:
         with open(args.table, "w") as f:
@@ -736,14 +744,43 @@ def dequant_full_model(args, torch, _capi, synth):
 
 
 
+def _llama2_7b_config():
+    from transformers import LlamaConfig
+    return LlamaConfig(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
+                       num_key_value_heads=32, vocab_size=32000, max_position_embeddings=4096, rms_norm_eps=1e-5,
+                       tie_word_embeddings=False)
+
+
+def decode_summary(torch, prompt_len=128, new_tokens=96):
+    """tokens/s of the graph-replayed decode step on a random-init Llama-2-7B-shaped model after a
+    128-token prompt, at 3 and 8 bits (the full sweep is --workload llama2_7b_decode)."""
+    from any_precision_amd import AnyPrecisionForCausalLM, GraphDecoder
+    model = AnyPrecisionForCausalLM.from_config(_llama2_7b_config(), seed=0, device="cuda")
+    dec = GraphDecoder(model, max_len=prompt_len + new_tokens + 8)
+    ids = torch.randint(0, 32000, (prompt_len,), generator=torch.Generator().manual_seed(0)).cuda()
+    rows = []
+    for b in (3, 8):
+        dec.prefill(ids, b)
+        dec.capture(b)
+        dec.decode(8, b)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.decode(new_tokens - 9, b)
+        torch.cuda.synchronize()
+        tok_s = (new_tokens - 9) / (time.perf_counter() - t0)
+        rows.append({"w_bits": b, "tokens_per_s": round(tok_s, 1), "ms_per_token": round(1e3 / tok_s, 3)})
+    del dec, model
+    torch.cuda.empty_cache()
+    return {"workload": f"greedy decode of {new_tokens} tokens after a {prompt_len}-token prompt, batch 1, 32 layers / hidden "
+                        "4096 / FFN 11008 / 32 heads / vocab 32000, random-init, decode step replayed from one HIP graph",
+            "per_w_bits": rows}
+
+
 def decode_tokens(args, torch, _capi, synth):
     """Batch-1 greedy decoding, random-init Llama-2-7B-shaped model: tokens/s per w_bits, the decode
     step replayed from a HIP graph; beside it the 224 GEMVs of a token alone and the eager loop."""
-    from transformers import LlamaConfig
     from any_precision_amd import AnyPrecisionForCausalLM, GraphDecoder
-    cfg = LlamaConfig(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
-                      num_key_value_heads=32, vocab_size=32000, max_position_embeddings=4096, rms_norm_eps=1e-5,
-                      tie_word_embeddings=False)
+    cfg = _llama2_7b_config()
     model = AnyPrecisionForCausalLM.from_config(cfg, seed=0, device="cuda")
     prompt_len, new_tokens = 128, 256
     dec = GraphDecoder(model, max_len=prompt_len + new_tokens + 8)
@@ -813,7 +850,7 @@ def decode_tokens(args, torch, _capi, synth):
         "data": "synthetic (random-init weights, random prompt ids)",
         "config": {"workload": f"greedy decode of {new_tokens} tokens after a {prompt_len}-token prompt, batch 1, "
                                "32 layers / hidden 4096 / FFN 11008 / 32 heads / vocab 32000; decode step replayed "
-                               "from one HIP graph, 9 launches per layer, all this library's (7 linears in 5 launches, "
+                               "from one HIP graph, 8 launches per layer, all this library's (7 linears in 4 launches, "
                                "add + RMSNorm twice, rotary + cache append + attention, SiLU * up); embedding, head "
                                "and argmax are PyTorch ops"},
         "per_w_bits": rows}))
