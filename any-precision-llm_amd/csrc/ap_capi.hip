@@ -7,6 +7,7 @@
 #include "ap_decode.hpp"
 #include "ap_dequant.hpp"
 #include "ap_gemm_launch.hpp"
+#include "ap_gemmw_launch.hpp"
 #include "ap_gemv4_launch.hpp"
 #include "ap_gemv_launch.hpp"
 #include "ap_gemvf_launch.hpp"
@@ -40,6 +41,8 @@ enum {
     kGemvFine,          // fine-grained row-pair GEMV: 0 never, 1 where it pays, 2 wherever it fits
     kGemvPersist,       // persistent row-loop GEMV: 0 never, 1 where it pays, 2 wherever it fits
     kGemvPersistWaves,  // waves per CU the persistent GEMV grid aims for
+    kGemmWalk,          // row-walking fused GEMM: 0 never, 1 where it pays, 2 wherever it fits
+    kGemmWalkWgs,       // workgroups per CU its grid aims for
     kKnobCount
 };
 Knob g_knobs[kKnobCount] = {
@@ -47,6 +50,7 @@ Knob g_knobs[kKnobCount] = {
     {"matmul_mfma_from", 5},      {"gemm_split", 0},     {"matmul_mfma4", 1}, {"gemv4_groups", 0},
     {"gemm_rb2", 1},              {"gemv_stream", 1},    {"gemv_stream_waves", 24},
     {"gemv_fine", 1},             {"gemv_persist", 1},   {"gemv_persist_waves", 8},
+    {"gemm_walk", 1},             {"gemm_walk_wgs", 1},
 };
 inline int knob(int k) { return __atomic_load_n(&g_knobs[k].value, __ATOMIC_RELAXED); }
 
@@ -296,11 +300,56 @@ int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits, int *wpl, int *segm
 
 namespace {
 
+// The row-walking fused GEMM serves up to 32 activation rows on rows of a multiple of 128 elements that its
+// K-split waves cover with one step of 512 elements each (two steps at up to 16 activation rows and 5 bits:
+// beyond, the double-buffered planes no longer fit the registers).
+bool gemmw_geometry(int M, int N, int K, int w_bits, GemmwGeometry *geo) {
+    const int W = K >> 5;
+    if (M < 1 || M > kGemmwMaxM || (W & 3) != 0 || N < 16) return false;
+    const int steps = (W + 15) / 16;
+    const int mb = (M + 15) / 16, spw = steps <= kGemmMaxSplit ? 1 : 2;
+    if (steps > 2 * kGemmMaxSplit || mb * spw > 2 || (spw == 2 && w_bits > 5)) return false;
+    const int ks = (steps + spw - 1) / spw;
+    if (ks < 4) return false;
+    if ((long long)M * K * 2 > 0xffffffffLL) return false;
+    const int nblocks = (N + 15) / 16;
+    int per_cu = knob(kGemmWalkWgs);
+    if (per_cu < 1) per_cu = 1;
+    const long long wgs = (long long)cu_count() * per_cu;
+    const long long rounds = (nblocks + wgs - 1) / wgs;
+    geo->mb = mb;
+    geo->spw = spw;
+    geo->ks = ks;
+    geo->grid = (int)((nblocks + rounds - 1) / rounds);  // every workgroup walks `rounds` blocks (the last ones one fewer)
+    return true;
+}
+
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
 int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
              int w_bits, hipStream_t st) {
     // the kernel addresses the activations with 32-bit byte offsets
     if ((long long)M * K * 2 > 0xffffffffLL) return AP_ELIMIT;
+    {
+        GemmwGeometry wgeo;
+        const int mode = knob(kGemmWalk);
+        // Where it pays (measured on 11008 / 14336 x 4096 and 28672 x 8192; 5-18 %): linears with at least 2.5
+        // blocks of rows per CU to walk, at 17..32 activation rows or at 8 bits with one step per wave, and from 9
+        // rows on with two.  Elsewhere the one-shot kernels are as fast or faster (fewer rows: nothing to walk; fewer
+        // activation rows at low bit-widths: their short waves hide the lookup latency better).
+        const bool pays = N >= 40 * cu_count() && (gemmw_geometry(M, N, K, w_bits, &wgeo)) &&
+                          (wgeo.spw == 1 ? (M > 16 || w_bits == 8) : M > 8);
+        if (mode > 0 && (mode >= 2 ? gemmw_geometry(M, N, K, w_bits, &wgeo) : pays)) {
+            switch (w_bits) {
+                case 3: launch_gemmw<3>(wgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 4: launch_gemmw<4>(wgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 5: launch_gemmw<5>(wgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 6: launch_gemmw<6>(wgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 7: launch_gemmw<7>(wgeo, x, qweight, lut, out, M, N, K, st); break;
+                default: launch_gemmw<8>(wgeo, x, qweight, lut, out, M, N, K, st); break;
+            }
+            return launch_status();
+        }
+    }
     GemmGeometry geo;
     geo.mb = (M + 15) / 16;
     const int W = K >> 5;

@@ -146,3 +146,45 @@ def test_two_weight_row_blocks_per_workgroup_give_the_same_bits(ext, oracle):
                 with _capi.tuning(gemm_rb2=0):
                     plain = ext.gemm_kbit(xg, q, luts[b], b)
                 assert torch.equal(plain.view(torch.int16), forced.view(torch.int16)), (N, K, b, M)
+
+
+def test_row_walking_kernel_agrees_with_the_oracle(ext, oracle):
+    """Wide linears at up to 32 activation rows run a variant whose workgroups walk the blocks of weight rows
+    with their activations held in registers; the knob gemm_walk = 2 forces it wherever it fits (rows of a
+    multiple of 128 elements, 4 to 16 steps of 512), on shapes small enough for the oracle: ragged row counts,
+    a partial last step (K = 2176, 6272), one and two steps per wave (K = 8192: up to 5 bits), more blocks
+    than workgroups (gemm_walk_wgs = 1 with 4112 rows on 256 CUs).  Also that it really is another kernel:
+    with the knob at 0 the same call gives the one-shot kernel's result, within rounding of it."""
+    from any_precision_amd import _capi
+    shapes = ((48, 2048), (100, 4096), (77, 2176), (40, 6272), (33, 8192), (4112, 2048))
+    for N, K in shapes:
+        L = make(N, K, seed=N + K)
+        q, luts = layer_to_gpu(L)
+        for b in range(3, 9):
+            for M in (1, 8, 16, 17, 32):
+                if K > 4096 and (b > 5 or M > 16):
+                    continue                     # two steps per wave exist up to 5 bits and 16 rows
+                print(f"row walk N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                with _capi.tuning(gemm_walk=2):
+                    walked = ext.gemm_kbit(xg, q, luts[b], b)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                assert_close_gemv(walked, want, f"N={N} K={K} b={b} M={M}")
+                with _capi.tuning(gemm_walk=0):
+                    plain = ext.gemm_kbit(xg, q, luts[b], b)
+                assert_close_gemv(plain, want, f"one-shot N={N} K={K} b={b} M={M}")
+
+
+def test_row_walking_kernel_on_a_wide_linear_by_default(ext, oracle):
+    """14336 x 4096 at 8 bits and at 17..32 rows takes the walking kernel by the default rule; a slice of its
+    outputs against the oracle on the same rows."""
+    N, K = 14336, 4096
+    L = make(N, K, seed=9)
+    q, luts = layer_to_gpu(L)
+    rows = np.r_[0:40, 7000:7040, N - 40:N]
+    for b, M in ((8, 5), (8, 16), (3, 32), (5, 20)):
+        print(f"row walk default N={N} K={K} b={b} M={M}", flush=True)
+        x, xg = _x(M, K, seed=M)
+        got = ext.gemm_kbit(xg, q, luts[b], b)
+        _, want = oracle.matmul_kbit(x, L.qweight[:, rows], L.luts[b][rows], b, return_f64=True)
+        assert_close_gemv(got[:, torch.from_numpy(rows).cuda()], want, f"N={N} K={K} b={b} M={M}")
