@@ -790,6 +790,20 @@ def decode_tokens(args, torch, _capi, synth):
     lib = _capi.lib
     side = torch.cuda.Stream()
     rows = []
+    if args.eager:
+        # for a kernel trace: the prompt, then 16 tokens launched one kernel at a time, at 3 and 8 bits
+        for b in (3, 8):
+            dec.prefill(ids, b)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dec.decode(16, b, use_graph=False)
+            torch.cuda.synchronize()
+            rows.append({"w_bits": b, "eager_tokens_per_s": round(16 / (time.perf_counter() - t0), 1)})
+        print(json.dumps({"metric": "batch-1 decode tokens/s, eager launches (for profiling)", "value": None, "unit": "tokens/s",
+                          "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "data": "synthetic",
+                          "config": {"workload": f"{prompt_len}-token prompt + 16 eager tokens, Llama-2-7B-shaped model"},
+                          "per_w_bits": rows}))
+        return
     for b in BITS:
         dec.prefill(ids, b)
         dec.capture(b)
