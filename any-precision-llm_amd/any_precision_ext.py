@@ -6,8 +6,8 @@ signatures, same result shapes and dtypes.
     dequant_kbit(qweight, lut, w_bits)    -> Tensor   main.cu:60-91
 
 plus one op the reference does not have, ``gemm_kbit(in, qweight, lut, w_bits)``: the
-fused dequant -> MFMA GEMM for up to ``GEMM_MAX_M`` activation rows (the reference's
-``dequant_kbit`` + ``torch.matmul`` branch, AnyPrecisionLinear.py:60-62, in one launch).
+fused dequant -> MFMA GEMM (the reference's ``dequant_kbit`` + ``torch.matmul`` branch,
+AnyPrecisionLinear.py:60-62, in one launch per ``GEMM_MAX_M`` activation rows).
 
 The ops validate their arguments, allocate the result with torch and hand raw
 device pointers plus torch's current HIP stream to libanyprec_hip.so.  Where
@@ -126,8 +126,8 @@ def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int, concat: bo
 
 
 def gemm_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:
-    """fp16 in_.shape[:-1] + [N] = in_ @ dequant(qweight, lut, w_bits).T for 1 <= M <= GEMM_MAX_M rows,
-    without materialising the fp16 weight."""
+    """fp16 in_.shape[:-1] + [N] = in_ @ dequant(qweight, lut, w_bits).T without materialising the fp16
+    weight; one launch per GEMM_MAX_M rows."""
     N, K = _check_weight(qweight, lut, w_bits, "gemm_kbit")
     if in_.dtype != torch.float16:
         raise ValueError(f"gemm_kbit: input must be float16, got {in_.dtype}")
@@ -136,8 +136,8 @@ def gemm_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bit
     if in_.dim() < 1 or in_.shape[-1] != K:
         raise ValueError(f"gemm_kbit: input last dim must be K={K}, got {tuple(in_.shape)}")
     M = in_.numel() // K
-    if M < 1 or M > GEMM_MAX_M:
-        raise ValueError(f"gemm_kbit: batch M={M} outside 1..{GEMM_MAX_M}; use dequant_kbit + matmul beyond")
+    if M < 1:
+        raise ValueError("gemm_kbit: empty batch")
     if not in_.is_contiguous():
         raise ValueError("gemm_kbit: input must be contiguous")
     with torch.cuda.device(qweight.device):

@@ -604,10 +604,18 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     if (!x || !qweight || !lut || !out) return AP_ENULL;
     const int rc = check_common(N, K, w_bits);
     if (rc != AP_OK) return rc;
-    if (M < 1 || M > kGemmMaxM) return AP_EBATCH;
+    if (M < 1) return AP_EBATCH;
     if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
     drain_stale_error();
-    return run_gemm(x, qweight, lut, out, M, N, K, w_bits, static_cast<hipStream_t>(stream));
+    // one launch serves up to kGemmMaxM activation rows; more go in chunks of that many, in order (the planes
+    // are re-read per chunk; row offsets of 128 rows keep x and out 16-byte aligned for every K and N that passed)
+    for (int m0 = 0; m0 < M; m0 += kGemmMaxM) {
+        const int rows = M - m0 < kGemmMaxM ? M - m0 : kGemmMaxM;
+        const int r = run_gemm(x + (size_t)m0 * K, qweight, lut, out + (size_t)m0 * N, rows, N, K, w_bits,
+                               static_cast<hipStream_t>(stream));
+        if (r != AP_OK) return r;
+    }
+    return AP_OK;
 }
 
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N,

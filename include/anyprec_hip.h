@@ -72,11 +72,14 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
                          const uint16_t *const *lut, uint16_t *const *out, const int *N,
                          int M, int K, int w_bits, void *stream);
 
-/* Fused dequant -> MFMA GEMM, 1 <= M <= 128: out[M,N] = x[M,K] . dequant(qweight, lut)^T
+/* Fused dequant -> MFMA GEMM, M >= 1: out[M,N] = x[M,K] . dequant(qweight, lut)^T
  * without materialising the fp16 weight.  No single counterpart in the reference: it is the
  * M > 8 branch of AnyPrecisionLinear.forward (AnyPrecisionLinear.py:60-62: dequant_kbit,
- * main.cu:60-91, then torch.matmul) fused (one launch; more than 32 rows may run as launches
- * of 32 rows each, in order, on the same stream).  fp32 accumulation, fp16 result. */
+ * main.cu:60-91, then torch.matmul) fused.  One launch serves up to 128 activation rows (more
+ * than 32 may run as launches of 32 rows each); beyond 128 the call issues one launch per 128
+ * rows, in order, on the same stream, re-reading the planes for each -- correct for every M, but
+ * from a few hundred rows on dequant + a library GEMM is the faster pair.  fp32 accumulation,
+ * fp16 result. */
 int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int M, int N, int K, int w_bits, void *stream);
 

@@ -1,4 +1,4 @@
-"""gemm_kbit (fused dequant -> MFMA GEMM, M up to 128) on the GPU against the oracle,
+"""gemm_kbit (fused dequant -> MFMA GEMM, up to 128 rows per launch) on the GPU against the oracle,
 through the C ABI.  Tolerance: 1e-2 relative (normwise and against max |y|)."""
 import numpy as np
 import pytest
@@ -95,11 +95,17 @@ def test_matches_gemv_and_is_deterministic(ext):
     assert y3.shape == (2, 4, N) and torch.equal(y3.reshape(8, N).view(torch.int16), a.view(torch.int16))
 
 
-def test_batch_limit_and_errors(ext):
-    L = make(16, 64, seed=0)
+def test_more_than_128_rows_go_in_chunks_and_errors(ext, oracle):
+    L = make(40, 1056, seed=0)
     q, luts = layer_to_gpu(L)
-    with pytest.raises(ValueError, match="1..128"):
-        ext.gemm_kbit(torch.zeros((129, 64), dtype=torch.float16, device="cuda"), q, luts[3], 3)
+    for b, M in ((3, 129), (8, 300), (5, 512)):
+        print(f"gemm chunks b={b} M={M}", flush=True)
+        x, xg = _x(M, 1056, seed=M)
+        got = ext.gemm_kbit(xg, q, luts[b], b)
+        _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+        assert_close_gemv(got, want, f"b={b} M={M}")
+    with pytest.raises(ValueError, match="empty"):
+        ext.gemm_kbit(torch.zeros((0, 1056), dtype=torch.float16, device="cuda"), q, luts[3], 3)
     with pytest.raises(ValueError, match="float16"):
         ext.gemm_kbit(torch.zeros((16, 64), dtype=torch.float32, device="cuda"), q, luts[3], 3)
 
