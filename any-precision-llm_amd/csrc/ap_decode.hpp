@@ -145,6 +145,19 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(
     }
     __syncthreads();
 
+    // ---- the first value rows this lane will need are requested now: they do not depend on the scores, and the
+    // score pass and the softmax then hide their latency (LPK lanes per key, 8 dims = 16 bytes each)
+    constexpr int PF = 6;  // steps of NW * KPW keys held in registers (384 keys at HD = 128); later ones load in place
+    const int dl = lane % LPK, sub = lane / LPK;
+    const half_t *vbase = vcache + (size_t)kvh * max_len * HD + dl * DPT;
+    half8_t vpre[PF];
+#pragma unroll
+    for (int it = 0; it < PF; it++) {
+        const int j = wave * KPW + sub + it * NW * KPW;
+        vpre[it] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        if (j < pos) vpre[it] = *reinterpret_cast<const half8_t *>(vbase + (size_t)j * HD);
+    }
+
     // ---- scores against the cached keys: four lanes per key
     {
         const int quad = tid >> 2, part = tid & 3;
@@ -152,6 +165,7 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(
 #pragma unroll
         for (int d = 0; d < DPL; d++) qreg[d] = q_s[part * DPL + d];
         const half_t *kbase = kcache + (size_t)kvh * max_len * HD + part * DPL;
+#pragma unroll 4
         for (int j0 = 0; j0 < pos; j0 += kAttnThreads / 4) {
             const int j = j0 + quad;
             float s = 0.f;
@@ -204,15 +218,25 @@ __global__ __launch_bounds__(kAttnThreads) void decode_attention_kernel(
 #pragma unroll
     for (int w = 0; w < NW; w++) l += red[1][w];
 
-    // ---- weighted sum of the values: LPK lanes per key, 8 dims (16 bytes) each
+    // ---- weighted sum of the values
     {
-        const int dl = lane % LPK, sub = lane / LPK;
         float acc[DPT];
 #pragma unroll
         for (int e = 0; e < DPT; e++) acc[e] = 0.f;
-        const half_t *vbase = vcache + (size_t)kvh * max_len * HD + dl * DPT;
+#pragma unroll
+        for (int it = 0; it < PF; it++) {  // the prefetched rows (zeros past pos, and a zero weight past n)
+            const int j = wave * KPW + sub + it * NW * KPW;
+            const float p = j < n ? sc[j] : 0.f;
+            if (j == pos) {
+#pragma unroll
+                for (int e = 0; e < DPT; e++) acc[e] += p * vn_s[dl * DPT + e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < DPT; e++) acc[e] += p * (float)vpre[it][e];
+            }
+        }
 #pragma unroll 4
-        for (int j = wave * KPW + sub; j < n; j += NW * KPW) {
+        for (int j = wave * KPW + sub + PF * NW * KPW; j < n; j += NW * KPW) {
             const float p = sc[j];
             if (j < pos) {
                 const half8_t v = *reinterpret_cast<const half8_t *>(vbase + (size_t)j * HD);
