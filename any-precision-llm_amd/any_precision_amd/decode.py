@@ -6,9 +6,9 @@ Hugging Face loop (demo.py:59-80), which at batch 1 is bound by Python and launc
 not by the kernels.  Here one decode step -- embedding, 32 x (norm, q/k/v GEMV, rotary,
 cache write, attention over a static cache, o GEMV, norm, gate/up GEMV, SiLU, down GEMV),
 final norm, head, argmax, position increment -- is recorded once per precision and replayed
-per token: no host work between tokens.  With ``fused_ops`` (the default) a layer is 8 launches, all
-of this library: the seven linears in four (q/k/v and gate/up as one grouped launch each), residual add +
-RMSNorm twice, rotary + cache append + attention in one kernel, SiLU * up.  Without it everything
+per token: no host work between tokens.  With ``fused_ops`` (the default) a layer is 7 launches, all
+of this library: the seven linears in four (q/k/v as one grouped launch; gate and up as one launch that
+also applies SiLU(gate) * up), residual add + RMSNorm twice, rotary + cache append + attention in one kernel.  Without it everything
 but the linears is stock PyTorch ops, as in the reference (19 launches per layer); that path also
 serves the prompt and is what the fused one is tested against.
 
@@ -23,7 +23,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _capi
-from .linear import forward_group
+from .linear import forward_group, forward_swiglu
 
 
 def _rope(x, cos, sin_signed):
@@ -149,7 +149,7 @@ class GraphDecoder:
         return F.linear(h, self.head)
 
     def _forward_fused(self, precision):
-        """The token self.tok at cache row self.pos through the network -> logits [1, vocab]; 8 launches per layer."""
+        """The token self.tok at cache row self.pos through the network -> logits [1, vocab]; 7 launches per layer."""
         lib, st = _capi.lib, torch.cuda.current_stream(self.dev).cuda_stream
         H, eps = self.cfg.hidden_size, float(self.eps)
         scale = 1.0 / math.sqrt(self.hd)
@@ -172,11 +172,11 @@ class GraphDecoder:
                                                 self.f_ctx.data_ptr(), self.nh, self.nkv, self.hd, self.max_len, scale, st),
                         "ap_decode_attention")
             add_norm(att.o_proj(self.f_ctx, precision=precision), layer.post_attention_layernorm.weight)
-            if self.group_launches:
-                gate, up = forward_group((layer.mlp.gate_proj, layer.mlp.up_proj), self.f_x, precision)
+            if self.group_launches:      # gate, up and the activation function in one launch
+                forward_swiglu(layer.mlp.gate_proj, layer.mlp.up_proj, self.f_x, precision, out=self.f_act)
             else:
                 gate, up = layer.mlp.gate_proj(self.f_x, precision=precision), layer.mlp.up_proj(self.f_x, precision=precision)
-            _capi.check(lib.ap_silu_mul(gate.data_ptr(), up.data_ptr(), self.f_act.data_ptr(), gate.numel(), st), "ap_silu_mul")
+                _capi.check(lib.ap_silu_mul(gate.data_ptr(), up.data_ptr(), self.f_act.data_ptr(), gate.numel(), st), "ap_silu_mul")
             delta = layer.mlp.down_proj(self.f_act, precision=precision)
         add_norm(delta, self.final_norm)
         return F.linear(self.f_x, self.head)

@@ -14,9 +14,9 @@ import torch
 import torch.nn as nn
 
 try:
-    from any_precision_ext import matmul_kbit, matmul_kbit_group, dequant_kbit, gemm_kbit, GEMM_MAX_M
+    from any_precision_ext import matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, GEMM_MAX_M
 except ModuleNotFoundError:
-    matmul_kbit, matmul_kbit_group, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, None, 0
+    matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, None, None, 0
 
 
 def fused_gemm_pays(rows: int, out_features: int, w_bits: int) -> bool:
@@ -51,6 +51,25 @@ def forward_group(modules, x, precision=None, concat=False):
         if m.bias is not None:
             o += m.bias
     return torch.cat(res, dim=-1) if concat else res
+
+
+def forward_swiglu(gate, up, x, precision=None, out=None):
+    """``silu(gate(x)) * up(x)`` for two bias-free linears of one shape: up to 4 activation rows (and rows of at most
+    32768 elements) in ONE launch with the activation applied before the store; otherwise the two GEMVs (one grouped
+    launch where possible) and the product in PyTorch ops."""
+    rows = x.numel() // x.shape[-1]
+    w_bits = gate.precision if precision is None else precision
+    fits = (rows <= 4 and gate.bias is None and up.bias is None and gate.in_features <= 32768
+            and (gate.in_features, gate.out_features) == (up.in_features, up.out_features))
+    if fits:
+        return matmul_kbit_swiglu(x.contiguous(), gate.qweight, gate._buffers[f"lut{w_bits}"], up.qweight,
+                                  up._buffers[f"lut{w_bits}"], w_bits, out=out)
+    g, u = forward_group((gate, up), x, w_bits)
+    res = torch.nn.functional.silu(g) * u
+    if out is not None:
+        out.copy_(res.view_as(out))
+        return out
+    return res
 
 
 class AnyPrecisionLinear(nn.Module):

@@ -22,7 +22,7 @@ import torch
 
 from any_precision_amd import _capi
 
-__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "matmul_kbit_group", "GEMM_MAX_M"]
+__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "matmul_kbit_group", "matmul_kbit_swiglu", "GEMM_MAX_M"]
 
 GEMM_MAX_M = _capi.GEMM_MAX_M
 
@@ -123,6 +123,33 @@ def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int, concat: bo
     if concat:
         return joint if joint is not None else torch.cat(outs, dim=-1)
     return outs
+
+
+def matmul_kbit_swiglu(in_: torch.Tensor, qweight_gate, lut_gate, qweight_up, lut_up, w_bits: int, out=None) -> torch.Tensor:
+    """``silu(matmul_kbit(in_, gate)) * matmul_kbit(in_, up)`` for 1..4 activation rows in one launch, fp32 until the
+    store.  No counterpart in the reference (its ``fuse_layers`` hook is a stub, AnyPrecisionForCausalLM.py:168-172)."""
+    N, K = _check_weight(qweight_gate, lut_gate, w_bits, "matmul_kbit_swiglu")
+    if _check_weight(qweight_up, lut_up, w_bits, "matmul_kbit_swiglu") != (N, K):
+        raise ValueError("matmul_kbit_swiglu: gate and up must have one shape")
+    if in_.dtype != torch.float16 or not in_.is_contiguous():
+        raise ValueError("matmul_kbit_swiglu: input must be contiguous float16")
+    if in_.device != qweight_gate.device or in_.device != qweight_up.device:
+        raise ValueError("matmul_kbit_swiglu: input and weights must be on one device")
+    if in_.dim() < 1 or in_.shape[-1] != K:
+        raise ValueError(f"matmul_kbit_swiglu: input last dim must be K={K}, got {tuple(in_.shape)}")
+    M = in_.numel() // K
+    if M < 1 or M > 4:
+        raise ValueError(f"matmul_kbit_swiglu: batch M={M} outside 1..4")
+    with torch.cuda.device(in_.device):
+        if out is None:
+            out = torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device)
+        elif out.dtype != torch.float16 or not out.is_contiguous() or out.numel() != M * N or out.device != in_.device:
+            raise ValueError("matmul_kbit_swiglu: out must be a contiguous float16 tensor of M x N elements on the input's device")
+        rc = _lib.ap_matmul_kbit_swiglu(in_.data_ptr(), qweight_gate.data_ptr(), lut_gate.data_ptr(), qweight_up.data_ptr(),
+                                        lut_up.data_ptr(), out.data_ptr(), M, N, K, w_bits,
+                                        torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "matmul_kbit_swiglu")
+    return out
 
 
 def gemm_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:

@@ -599,6 +599,44 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
 
 extern "C" {
 
+int ap_matmul_kbit_swiglu(const uint16_t *x, const uint32_t *qweight_gate, const uint16_t *lut_gate,
+                          const uint32_t *qweight_up, const uint16_t *lut_up, uint16_t *out, int M, int N, int K, int w_bits,
+                          void *stream) {
+    if (!x || !qweight_gate || !lut_gate || !qweight_up || !lut_up || !out) return AP_ENULL;
+    const int rc = check_common(N, K, w_bits);
+    if (rc != AP_OK) return rc;
+    if (M < 1 || M > 4) return AP_EBATCH;
+    if (!aligned16(x) || !aligned16(qweight_gate) || !aligned16(lut_gate) || !aligned16(qweight_up) || !aligned16(lut_up))
+        return AP_EALIGN;
+    GemvGeometry geo;
+    geo.wpl = 1;
+    geo.S = ((K >> 5) + kWave - 1) / kWave;
+    geo.R = 2;
+    geo.grid = N;  // one workgroup per (gate row, up row) pair
+    if (geo.S > kGemvMaxSeg) return AP_ELIMIT;
+    GemvMembers mem;
+    memset(&mem, 0, sizeof mem);
+    mem.qweight[0] = qweight_gate;
+    mem.qweight[1] = qweight_up;
+    mem.lut[0] = lut_gate;
+    mem.lut[1] = lut_up;
+    mem.out[0] = mem.out[1] = out;
+    mem.n[0] = mem.n[1] = N;
+    mem.wg_end[0] = mem.wg_end[1] = N;
+    mem.count = 2;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    drain_stale_error();
+    switch (w_bits) {
+        case 3: launch_gemv_pair<3>(M, geo, x, mem, K, st); break;
+        case 4: launch_gemv_pair<4>(M, geo, x, mem, K, st); break;
+        case 5: launch_gemv_pair<5>(M, geo, x, mem, K, st); break;
+        case 6: launch_gemv_pair<6>(M, geo, x, mem, K, st); break;
+        case 7: launch_gemv_pair<7>(M, geo, x, mem, K, st); break;
+        default: launch_gemv_pair<8>(M, geo, x, mem, K, st); break;
+    }
+    return launch_status();
+}
+
 int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
                  int w_bits, void *stream) {
     if (!x || !qweight || !lut || !out) return AP_ENULL;

@@ -186,8 +186,13 @@ __device__ __forceinline__ void row_dot(const typename WordVec<WPL>::type (&q)[B
 // One launch serves up to kGemvMaxGroup linears that share x, K and the bit-width (the
 // q/k/v or gate/up projections of a decoder layer): `mem` lists them and the workgroup
 // range of each; a plain call is a set of one.
-template <int BITS, int M, int WPL, int R, int THREADS>
+//
+// PAIR (R = 2 only): the two rows of a workgroup are row n of member 0 and row n of member 1 (two linears of
+// equal shape), and what is stored is silu(member 0) * member 1 -- the gate and up projections of a SwiGLU
+// MLP with their activation function, one output per row pair, nothing written in between.
+template <int BITS, int M, int WPL, int R, int THREADS, bool PAIR = false>
 __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K) {
+    static_assert(!PAIR || R == 2, "a pair is two rows");
     constexpr int NC = 1 << BITS;
     constexpr int MAXS = THREADS / kWave;
     typedef typename WordVec<WPL>::type wvec_t;
@@ -201,7 +206,7 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__rest
     int N = mem.n[0], wg0 = 0;
 #pragma unroll
     for (int g = 1; g < kGemvMaxGroup; g++) {
-        if (g < mem.count && (int)blockIdx.x >= mem.wg_end[g - 1]) {
+        if (!PAIR && g < mem.count && (int)blockIdx.x >= mem.wg_end[g - 1]) {
             qweight = mem.qweight[g];
             lut = reinterpret_cast<const half_t *>(mem.lut[g]);
             out = reinterpret_cast<half_t *>(mem.out[g]);
@@ -219,7 +224,11 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__rest
     const uint32_t w0 = (uint32_t)(s * kWave + lane) * WPL;
     const bool valid = w0 < (uint32_t)W;
     const uint32_t wl = valid ? w0 : 0u;  // lanes past the row end read word 0; their sums are dropped
-    const int row0 = ((int)blockIdx.x - wg0) * R;
+    const int row0 = PAIR ? (int)blockIdx.x : ((int)blockIdx.x - wg0) * R;
+    // row r of this workgroup: its number, its planes and its tables
+    auto row_of = [&](int r) { return PAIR ? row0 : min(row0 + r, N - 1); };
+    auto planes_of = [&](int r) { return PAIR ? mem.qweight[r] : qweight; };
+    auto tables_of = [&](int r) { return PAIR ? reinterpret_cast<const half_t *>(mem.lut[r]) : lut; };
 
     // Issue order matters: the tables first (tiny; staging them to LDS then overlaps the
     // plane loads -- issued last, the table was the last thing to arrive and cost 15-20 %),
@@ -229,11 +238,11 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__rest
     TableRegs<BITS> t[R];
 #pragma unroll
     for (int r = 0; r < R; r++)
-        if (s == r % S) t[r] = table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane);
+        if (s == r % S) t[r] = table_fetch<BITS>(tables_of(r) + (size_t)row_of(r) * NC, lane);
     wvec_t q[R][BITS];
 #pragma unroll
     for (int r = 0; r < R; r++) {
-        const uint32_t *p0 = qweight + (size_t)min(row0 + r, N - 1) * W;  // uniform per wave
+        const uint32_t *p0 = planes_of(r) + (size_t)row_of(r) * W;  // uniform per wave
 #pragma unroll
         for (int p = 0; p < BITS; p++)  // streamed once: non-temporal, so x and the tables keep their cache lines
             q[r][p] = __builtin_nontemporal_load(reinterpret_cast<const wvec_t *>(p0 + p * plane_stride + wl));
@@ -257,13 +266,19 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__rest
         for (int m = 0; m < M; m++) tot[r][m] = wave_sum(valid ? acc[m][0] + acc[m][1] : 0.f);
     });
 
+    auto swiglu = [](float gate, float up) { return gate / (1.f + __expf(-gate)) * up; };
     if (S == 1) {
         if (lane == kSumLane) {
+            if constexpr (PAIR) {
 #pragma unroll
-            for (int r = 0; r < R; r++)
+                for (int m = 0; m < M; m++) out[(size_t)m * N + row0] = (half_t)swiglu(tot[0][m], tot[R - 1][m]);
+            } else {
 #pragma unroll
-                for (int m = 0; m < M; m++)
-                    if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)tot[r][m];
+                for (int r = 0; r < R; r++)
+#pragma unroll
+                    for (int m = 0; m < M; m++)
+                        if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)tot[r][m];
+            }
         }
     } else {
         if (lane == kSumLane) {
@@ -274,7 +289,16 @@ __global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__rest
         }
         __syncthreads();
         const int tid = s * kWave + lane;
-        if (tid < R * M) {  // S >= 2 waves hold at least 128 threads >= R * M
+        if constexpr (PAIR) {
+            if (tid < M) {
+                float g = 0.f, u = 0.f;
+                for (int ss = 0; ss < S; ss++) {
+                    g += partial[(ss * R) * M + tid];
+                    u += partial[(ss * R + R - 1) * M + tid];
+                }
+                out[(size_t)tid * N + row0] = (half_t)swiglu(g, u);
+            }
+        } else if (tid < R * M) {  // S >= 2 waves hold at least 128 threads >= R * M
             const int m = tid % M, r = tid / M;
             float v = 0.f;
             for (int ss = 0; ss < S; ss++) v += partial[(ss * R + r) * M + m];

@@ -33,7 +33,31 @@ void launch_m(const GemvGeometry &geo, const half_t *x, const GemvMembers &mem, 
     launch_rows<BITS, M, 1, 2>(geo, x, mem, K, stream);
 }
 
+template <int BITS, int M>
+void launch_pair_m(const GemvGeometry &geo, const half_t *x, const GemvMembers &mem, int K, hipStream_t stream) {
+    const dim3 block(kWave, geo.S), grid(geo.grid);
+    if (geo.S <= 4)
+        gemv_kbit_kernel<BITS, M, 1, 2, 256, true><<<grid, block, 0, stream>>>(x, mem, K);
+    else if (geo.S <= 8)
+        gemv_kbit_kernel<BITS, M, 1, 2, 512, true><<<grid, block, 0, stream>>>(x, mem, K);
+    else
+        gemv_kbit_kernel<BITS, M, 1, 2, 1024, true><<<grid, block, 0, stream>>>(x, mem, K);
+}
+
 }  // namespace
+
+template <int BITS>
+void launch_gemv_pair(int M, const GemvGeometry &geo, const uint16_t *x, const GemvMembers &mem, int K, hipStream_t stream) {
+    const half_t *xh = reinterpret_cast<const half_t *>(x);
+    switch (M) {
+        case 1: return launch_pair_m<BITS, 1>(geo, xh, mem, K, stream);
+        case 2: return launch_pair_m<BITS, 2>(geo, xh, mem, K, stream);
+        case 3: return launch_pair_m<BITS, 3>(geo, xh, mem, K, stream);
+        default: return launch_pair_m<BITS, 4>(geo, xh, mem, K, stream);
+    }
+}
+
+template void launch_gemv_pair<AP_BITS>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
 
 template <int BITS>
 void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const GemvMembers &mem, int K, hipStream_t stream) {

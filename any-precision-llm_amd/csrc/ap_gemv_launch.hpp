@@ -33,6 +33,19 @@ template <int BITS>
 void launch_gemv(int M, const GemvGeometry &geo, const uint16_t *x, const GemvMembers &members, int K,
                  hipStream_t stream);
 
+// Launches gemv_kbit_kernel<BITS, M, 1, 2, *, true>: members 0 and 1 of `members` are two linears of n[0] rows
+// each (gate and up), out[0] receives silu(member 0) * member 1; geo.wpl = 1, geo.R = 2, geo.grid = n[0].  1 <= M <= 4.
+template <int BITS>
+void launch_gemv_pair(int M, const GemvGeometry &geo, const uint16_t *x, const GemvMembers &members, int K,
+                      hipStream_t stream);
+
+extern template void launch_gemv_pair<3>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv_pair<4>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv_pair<5>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv_pair<6>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv_pair<7>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+extern template void launch_gemv_pair<8>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
+
 extern template void launch_gemv<3>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
 extern template void launch_gemv<4>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);
 extern template void launch_gemv<5>(int, const GemvGeometry &, const uint16_t *, const GemvMembers &, int, hipStream_t);

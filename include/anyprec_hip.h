@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 4
+#define AP_ABI_VERSION 5
 
 enum {
     AP_OK = 0,
@@ -71,6 +71,17 @@ int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *l
 int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight,
                          const uint16_t *const *lut, uint16_t *const *out, const int *N,
                          int M, int K, int w_bits, void *stream);
+
+/* The gate and up projections of a SwiGLU MLP with their activation function, for 1 <= M <= 4 rows:
+ *     out[M,N] = silu(x . W_gate^T) * (x . W_up^T),   silu(v) = v / (1 + exp(-v)),
+ * two linears of equal shape [N,K] at the same w_bits, one launch, one rounding (fp32 until the store).
+ * The reference computes the two products with two matmul_kbit calls (main.cu:93-143) and leaves the
+ * activation to the Hugging Face MLP module it wraps (AnyPrecisionForCausalLM.py:88-97); its own
+ * fuse_layers hook is a stub (:168-172).  AP_EBATCH beyond 4 rows, AP_ELIMIT for rows longer than
+ * 32768 elements: call ap_matmul_kbit_group and ap_silu_mul there. */
+int ap_matmul_kbit_swiglu(const uint16_t *x, const uint32_t *qweight_gate, const uint16_t *lut_gate,
+                          const uint32_t *qweight_up, const uint16_t *lut_up, uint16_t *out,
+                          int M, int N, int K, int w_bits, void *stream);
 
 /* Fused dequant -> MFMA GEMM, M >= 1: out[M,N] = x[M,K] . dequant(qweight, lut)^T
  * without materialising the fp16 weight.  No single counterpart in the reference: it is the

@@ -70,6 +70,15 @@ def test_decode_step_argument_errors_need_no_gpu():
     assert L.ap_add_rmsnorm(fake, None, fake, fake, fake, 0, 128, 1e-5, None) == _capi.AP_ESHAPE
     assert L.ap_add_rmsnorm(fake, None, fake, fake, fake, 1, 100, 1e-5, None) == _capi.AP_ESHAPE
     assert L.ap_add_rmsnorm(fake, fake + 2, fake, fake, fake, 1, 128, 1e-5, None) == _capi.AP_EALIGN
+    sw = lambda **kw: L.ap_matmul_kbit_swiglu(*[kw.get(k, d) for k, d in (
+        ("x", fake), ("qg", fake), ("lg", fake), ("qu", fake), ("lu", fake), ("out", fake), ("M", 1), ("N", 8), ("K", 64),
+        ("b", 3), ("stream", None))])
+    assert sw(qu=None) == _capi.AP_ENULL
+    assert sw(M=5) == _capi.AP_EBATCH
+    assert sw(b=9) == _capi.AP_EBITS
+    assert sw(K=40) == _capi.AP_ESHAPE
+    assert sw(K=32 * 64 * 17) == _capi.AP_ELIMIT          # more than 16 waves per row
+    assert sw(lg=fake + 4) == _capi.AP_EALIGN
     assert L.ap_silu_mul(fake, None, fake, 64, None) == _capi.AP_ENULL
     assert L.ap_silu_mul(fake, fake, fake, 12, None) == _capi.AP_ESHAPE
     assert L.ap_silu_mul(fake, fake, fake + 4, 64, None) == _capi.AP_EALIGN

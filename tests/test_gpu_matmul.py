@@ -341,3 +341,27 @@ def test_non_finite_values_stay_where_they_belong(ext):
                 x2[1, -1] = float("inf")                   # last element of activation row 1
                 y = ext.matmul_kbit(x2, q, luts[b], b)
                 assert torch.isfinite(y[0]).all() and not torch.isfinite(y[1]).any()
+
+
+def test_gate_and_up_with_their_activation_in_one_launch(oracle):
+    """matmul_kbit_swiglu = silu(x W_gate^T) * (x W_up^T) from the oracle's float64 products; 1..4 rows, one and
+    several waves per row, ragged row counts, a tail chunk (K = 11008), every bit-width.  The single rounding makes
+    it closer to the float64 statement than the three-kernel path, so the usual 1e-2 bar holds with room."""
+    import any_precision_ext as ext
+    for N, K in ((33, 64), (100, 2048), (64, 4096), (40, 11008), (7, 8192)):
+        Lg, Lu = make(N, K, seed=N + K), make(N, K, seed=N + K + 1)
+        qg, lg = layer_to_gpu(Lg)
+        qu, lu = layer_to_gpu(Lu)
+        for b in range(3, 9):
+            for M in (1, 2, 3, 4):
+                print(f"swiglu N={N} K={K} b={b} M={M}", flush=True)
+                x = synth.make_x(M, K, seed=M)
+                xg = torch.from_numpy(x).cuda()
+                got = ext.matmul_kbit_swiglu(xg, qg, lg[b], qu, lu[b], b)
+                assert got.shape == (M, N) and got.dtype == torch.float16
+                _, g64 = oracle.matmul_kbit(x, Lg.qweight, Lg.luts[b], b, return_f64=True)
+                _, u64 = oracle.matmul_kbit(x, Lu.qweight, Lu.luts[b], b, return_f64=True)
+                want = g64 / (1.0 + np.exp(-g64)) * u64
+                assert_close_gemv(got, want, f"swiglu N={N} K={K} b={b} M={M}")
+    with pytest.raises(ValueError, match="1..4"):
+        ext.matmul_kbit_swiglu(torch.zeros((5, 8192), dtype=torch.float16, device="cuda"), qg, lg[3], qu, lu[3], 3)
