@@ -26,7 +26,9 @@ __device__ __forceinline__ float wave_max(float v) {
 // One workgroup per row of H elements (H % 8 == 0):
 //     s = h + delta (rounded to fp16, as an fp16 add; delta may be null), written to h_out;
 //     x_out = s * rsqrt(mean(s^2) + eps) * weight.
-// h_out may alias h.
+// h_out may alias h.  Rows of up to 8 * kNormThreads * kNormHeld elements (8192) stay in registers between the
+// two passes and the weight is requested before the reduction; longer rows re-read what they wrote.
+constexpr int kNormHeld = 4;
 __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const half_t *h, const half_t *delta,
                                                                    const half_t *__restrict__ weight, half_t *h_out,
                                                                    half_t *__restrict__ x_out, int H, float eps) {
@@ -37,8 +39,10 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const half_t 
     const half_t *dr = delta ? delta + row * H : nullptr;
     half_t *ho = h_out + row * H;
     const bool rewrite = dr != nullptr || ho != hr;
+    constexpr int STEP = kNormThreads * 8;
+    half8_t held[kNormHeld], wheld[kNormHeld];
     float ss = 0.f;
-    for (int i = tid * 8; i < H; i += kNormThreads * 8) {
+    auto summed = [&](int i) {
         half8_t a = *reinterpret_cast<const half8_t *>(hr + i);
         if (dr) {
             const half8_t b = *reinterpret_cast<const half8_t *>(dr + i);
@@ -48,7 +52,17 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const half_t 
         if (rewrite) *reinterpret_cast<half8_t *>(ho + i) = a;
 #pragma unroll
         for (int e = 0; e < 8; e++) ss += (float)a[e] * (float)a[e];
+        return a;
+    };
+#pragma unroll
+    for (int c = 0; c < kNormHeld; c++) {
+        const int i = tid * 8 + c * STEP;
+        if (i < H) {
+            wheld[c] = *reinterpret_cast<const half8_t *>(weight + i);
+            held[c] = summed(i);
+        }
     }
+    for (int i = tid * 8 + kNormHeld * STEP; i < H; i += STEP) summed(i);
     ss = wave_sum(ss);
     if ((tid & (kWave - 1)) == kSumLane) red[tid / kWave] = ss;
     __syncthreads();
@@ -56,15 +70,20 @@ __global__ __launch_bounds__(kNormThreads) void add_rmsnorm_kernel(const half_t 
 #pragma unroll
     for (int w = 0; w < kNormThreads / kWave; w++) total += red[w];
     const float rs = rsqrtf(total / (float)H + eps);
-    const half_t *src = rewrite ? ho : hr;  // every thread re-reads exactly what it wrote
-    for (int i = tid * 8; i < H; i += kNormThreads * 8) {
-        const half8_t a = *reinterpret_cast<const half8_t *>(src + i);
-        const half8_t w = *reinterpret_cast<const half8_t *>(weight + i);
+    auto scaled = [&](const half8_t &a, const half8_t &w, int i) {
         half8_t y;
 #pragma unroll
         for (int e = 0; e < 8; e++) y[e] = (half_t)((float)a[e] * rs * (float)w[e]);
         *reinterpret_cast<half8_t *>(x_out + row * H + i) = y;
+    };
+#pragma unroll
+    for (int c = 0; c < kNormHeld; c++) {
+        const int i = tid * 8 + c * STEP;
+        if (i < H) scaled(held[c], wheld[c], i);
     }
+    const half_t *src = rewrite ? ho : hr;  // every thread re-reads exactly what it wrote
+    for (int i = tid * 8 + kNormHeld * STEP; i < H; i += STEP)
+        scaled(*reinterpret_cast<const half8_t *>(src + i), *reinterpret_cast<const half8_t *>(weight + i), i);
 }
 
 // out = gate / (1 + exp(-gate)) * up over n elements (n % 8 == 0).
