@@ -102,6 +102,16 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // tail).  From M = 3 on the activations are the larger load: always two rows.
     int R = force_rows > 0 ? force_rows : (int)((rows * S + target_waves - 1) / (target_waves > 0 ? target_waves : 1));
     R = (R >= 2 || M > 2) ? 2 : 1;
+    // Four rows per workgroup (one activation row, one word per lane): the activations a wave holds then serve
+    // four rows, which halves their traffic through the L1 once more, at the price of half the waves.  Measured
+    // 3-6 % faster (two boxes, run-to-run noise about as large) on single linears of at least 28000 waves at up to
+    // 4 bits (14336 x 4096, 4096 x 14336) and, with rows of at least 8192 elements, at every bit-width
+    // (8192 x 8192, 28672 x 8192); equal or slower on the Llama-2-7B shapes, so those keep two.
+    if (M == 1 && wpl == 1) {
+        const long long waves = rows * S;
+        const bool pays = count == 1 && waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768));
+        if (force_rows == 4 || (force_rows <= 0 && pays)) R = 4;
+    }
     geo->wpl = wpl;
     geo->S = S;
     geo->R = R;

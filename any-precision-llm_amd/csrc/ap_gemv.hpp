@@ -174,7 +174,7 @@ __device__ __forceinline__ void row_dot(const typename WordVec<WPL>::type (&q)[B
     }
 }
 
-// The GEMV kernel.  A workgroup is the S waves of R consecutive rows (R = 1 or 2,
+// The GEMV kernel.  A workgroup is the S waves of R consecutive rows (R = 1, 2 or 4,
 // compile time).  Every wave issues all the global loads it will ever need -- the tables,
 // the planes of its R rows, its activations -- before it computes anything, so the
 // memory pipe is full from the first cycle and there is no loop-carried prefetch.  Every

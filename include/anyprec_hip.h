@@ -109,7 +109,7 @@ int ap_matmul_kbit_geometry(int M, int N, int K, int w_bits,
 /* Which kernel ap_matmul_kbit would launch for one linear (output taken to be 4-byte aligned), for
  * reports and tests.  Returns AP_OK or the argument errors of ap_matmul_kbit. */
 enum {
-    AP_ROUTE_DOT = 0,     /* gemv_kbit_kernel: one or two rows per workgroup, one word per lane         */
+    AP_ROUTE_DOT = 0,     /* gemv_kbit_kernel: one, two or four rows per workgroup                      */
     AP_ROUTE_STREAM = 1,  /* gemvp_kbit_kernel: row pairs, 16-byte plane loads, few long waves           */
     AP_ROUTE_FINE = 2,    /* gemvf_kbit_kernel: one workgroup per row pair, 8-byte plane loads           */
     AP_ROUTE_PERSIST = 3, /* gemvr_kbit_kernel: persistent row loop (only when forced)                   */

@@ -365,3 +365,27 @@ def test_gate_and_up_with_their_activation_in_one_launch(oracle):
                 assert_close_gemv(got, want, f"swiglu N={N} K={K} b={b} M={M}")
     with pytest.raises(ValueError, match="1..4"):
         ext.matmul_kbit_swiglu(torch.zeros((5, 8192), dtype=torch.float16, device="cuda"), qg, lg[3], qu, lu[3], 3)
+
+
+def test_four_rows_per_workgroup_agree_with_the_oracle(ext, oracle):
+    """At one activation row, long or many rows at low bit-widths run the dot-product kernel with four rows per
+    workgroup; the knob gemv_rows = 4 forces it on small shapes (row counts that are no multiple of 4, one to
+    seven waves per row, a tail chunk), and the geometry report shows where the default rule picks it."""
+    from any_precision_amd import _capi
+    for N, K in ((1, 64), (7, 2048), (33, 4096), (100, 11008), (18, 14336), (130, 1056)):
+        L = make(N, K, seed=N + K)
+        q, luts = layer_to_gpu(L)
+        for b in range(3, 9):
+            print(f"four rows N={N} K={K} b={b}", flush=True)
+            x, xg = _x(1, K, seed=b)
+            with _capi.tuning(gemv_rows=4, gemv_stream=0, gemv_fine=0):
+                assert _capi.matmul_geometry(1, N, K, b)["rows"] == 4
+                got = ext.matmul_kbit(xg, q, luts[b], b)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"N={N} K={K} b={b}")
+    assert _capi.matmul_geometry(1, 14336, 4096, 3)["rows"] == 4      # 28672 waves at 3 bits
+    assert _capi.matmul_geometry(1, 14336, 4096, 8)["rows"] == 2
+    assert _capi.matmul_geometry(1, 8192, 8192, 8)["rows"] == 4       # long rows: at every bit-width
+    assert _capi.matmul_geometry(1, 4096, 11008, 3)["rows"] == 2
+    assert _capi.matmul_geometry(1, 4096, 4096, 3)["rows"] == 1
+    assert _capi.matmul_geometry(2, 14336, 4096, 3)["rows"] == 2      # one activation row only
