@@ -5,7 +5,7 @@ Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]
 ``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
 ``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
 Batch dispatch: up to 8 activation rows -> ``matmul_kbit`` as in the reference (:60-64);
-9 .. 32 rows (.. 64 where ``fused_gemm_pays`` says so) -> the fused ``gemm_kbit``; beyond ->
+9 .. 32 rows (.. 64 or 128 where ``fused_gemm_pays`` says so) -> the fused ``gemm_kbit``; beyond ->
 ``dequant_kbit`` + ``torch.matmul`` as in the reference.
 """
 from __future__ import annotations
@@ -19,14 +19,17 @@ except ModuleNotFoundError:
     matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, None, None, 0
 
 
-def fused_gemm_pays(rows: int, out_features: int, w_bits: int) -> bool:
+def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int = 0) -> bool:
     """Whether the fused GEMM beats dequant_kbit + torch.matmul (measured on the Llama-2-7B / Llama-3-8B
     / 8192 x 8192 shapes, every bit-width): always up to 32 activation rows (1.3-2.6x at 16); up to 64
-    on linears of fewer than 8192 rows, and on larger ones at up to 5 bits.  Beyond, the re-read of
+    on linears of fewer than 8192 rows, and on larger ones at up to 5 bits; up to 128 on linears of fewer
+    than 8192 rows of at most 4096 elements (4096 x 4096: 33-35 us against 43).  Beyond, the re-read of
     the activations per block of weight rows costs more than materialising the weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
-    return rows <= min(64, GEMM_MAX_M) and (out_features < 8192 or w_bits <= 5)
+    if rows <= min(64, GEMM_MAX_M):
+        return out_features < 8192 or w_bits <= 5
+    return rows <= min(128, GEMM_MAX_M) and out_features < 8192 and 0 < in_features <= 4096
 
 
 def forward_group(modules, x, precision=None, concat=False):
@@ -125,7 +128,7 @@ class AnyPrecisionLinear(nn.Module):
         if rows <= 8:                                       # GEMV / skinny kernels (reference: :63-64)
             # the ops take dense row-major activations; a transposed or sliced view is copied (a no-op otherwise)
             y = matmul_kbit(x.contiguous(), self.qweight, table, w_bits)
-        elif fused_gemm_pays(rows, self.out_features, w_bits):
+        elif fused_gemm_pays(rows, self.out_features, w_bits, self.in_features):
             y = gemm_kbit(x.contiguous(), self.qweight, table, w_bits)   # fused dequant -> MFMA, weight never materialised
         else:                                               # reference: :60-62
             y = torch.matmul(x, dequant_kbit(self.qweight, table, w_bits).T)

@@ -55,4 +55,5 @@ def test_fused_gemm_dispatch_rule():
     from any_precision_amd.linear import fused_gemm_pays
     assert all(fused_gemm_pays(m, n, b) for m in (9, 32) for n in (4096, 14336) for b in (3, 8))
     assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6)
-    assert not fused_gemm_pays(65, 4096, 3)
+    assert not fused_gemm_pays(65, 4096, 3) and not fused_gemm_pays(65, 4096, 3, 11008) and not fused_gemm_pays(129, 4096, 3, 4096)
+    assert fused_gemm_pays(128, 4096, 8, 4096) and not fused_gemm_pays(128, 11008, 3, 4096)

@@ -36,7 +36,7 @@ def test_forward_every_branch_and_bias(oracle):
     m, sd = _module(L)
     bias = sd["bias"].numpy().astype(np.float64)
     for b in (3, 5, 8):
-        for M in (1, 8, 9, 32, 33, 64, 65, 130):      # GEMV | fused GEMM (to 64 rows here) | dequant + matmul
+        for M in (1, 8, 9, 32, 33, 64, 65, 128, 130): # GEMV | fused GEMM (to 128 rows here: 128 x 4096) | dequant + matmul
             x = synth.make_x(M, L.K, seed=M)
             y = m(torch.from_numpy(x).cuda(), precision=b)
             _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
