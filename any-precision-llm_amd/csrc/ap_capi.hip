@@ -107,9 +107,14 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // 3-6 % faster (two boxes, run-to-run noise about as large) on single linears of at least 28000 waves at up to
     // 4 bits (14336 x 4096, 4096 x 14336) and, with rows of at least 8192 elements, at every bit-width
     // (8192 x 8192, 28672 x 8192); equal or slower on the Llama-2-7B shapes, so those keep two.
+    // Launches of several linears (q/k/v: 3 x 4096 x 4096 = 24576 waves) measured differently from single ones of
+    // the same size: at 7-8 bits ONE row per workgroup is 8-15 % faster up to 32768 waves (more waves in flight
+    // for the lookups), at 3-4 bits FOUR rows are 3-6 % faster from 20000 waves on.
+    if (count > 1 && M == 1 && wpl == 1 && force_rows <= 0 && w_bits >= 7 && rows * S <= 32768) R = 1;
     if (M == 1 && wpl == 1) {
         const long long waves = rows * S;
-        const bool pays = count == 1 && waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768));
+        const bool pays = count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
+                                     : waves >= 20000 && w_bits <= 4;
         if (force_rows == 4 || (force_rows <= 0 && pays)) R = 4;
     }
     geo->wpl = wpl;
