@@ -107,10 +107,13 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // 3-6 % faster (two boxes, run-to-run noise about as large) on single linears of at least 28000 waves at up to
     // 4 bits (14336 x 4096, 4096 x 14336) and, with rows of at least 8192 elements, at every bit-width
     // (8192 x 8192, 28672 x 8192); equal or slower on the Llama-2-7B shapes, so those keep two.
-    // Launches of several linears (q/k/v: 3 x 4096 x 4096 = 24576 waves) measured differently from single ones of
-    // the same size: at 7-8 bits ONE row per workgroup is 8-15 % faster up to 32768 waves (more waves in flight
-    // for the lookups), at 3-4 bits FOUR rows are 3-6 % faster from 20000 waves on.
-    if (count > 1 && M == 1 && wpl == 1 && force_rows <= 0 && w_bits >= 7 && rows * S <= 32768) R = 1;
+    // At the highest bit-widths the lookups want more waves in flight: ONE row per workgroup up to 32768 waves is
+    // 8-15 % faster at 7-8 bits for launches of several linears (q/k/v: 3 x 4096 x 4096 = 24576 waves) and 2-7 %
+    // faster at 8 bits for single wide ones of short rows (11008 / 14336 x 4096).  At 3-4 bits launches of several
+    // linears are 3-6 % faster with FOUR rows from 20000 waves on.
+    if (M == 1 && wpl == 1 && force_rows <= 0 && rows * S <= 32768 &&
+        (count > 1 ? w_bits >= 7 : (w_bits == 8 && K < 8192)))
+        R = 1;
     if (M == 1 && wpl == 1) {
         const long long waves = rows * S;
         const bool pays = count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
@@ -554,8 +557,9 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     //  - row-streaming kernel (fewest waves and instructions): 3 bits at batch 1 on linears of >= 8192
     //    rows of <= 4096 elements (gate/up of the 7B/8B models: 3-5 %), 3-4 bits at batch 2 on rows of
     //    >= 8192 elements (10-14 %);
-    //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-8 bits at batch 1 on the
-    //    same wide linears (3-6 %), 6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %).
+    //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-7 bits at batch 1 on the
+    //    same wide linears (3-6 %; at 8 bits gemv_kbit_kernel with one row per workgroup is faster still),
+    //    6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %).
     // Mode 2 of a knob forces its kernel wherever it fits (tests, sweeps); mode 0 switches it off.
     const int persist_mode = knob(kGemvPersist), fine_mode = knob(kGemvFine), stream_mode = knob(kGemvStream);
     bool fits_r = true, fits_f = true, fits_p = true;
@@ -572,7 +576,7 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         const bool wide = N[0] >= 8192 && K <= 4096;
         if (stream_mode == 1 && fits_p && ((M == 1 && wide && w_bits == 3) || (M == 2 && K >= 8192 && w_bits <= 4)))
             return all(AP_ROUTE_STREAM);
-        if (fine_mode == 1 && fits_f && ((M == 1 && wide && w_bits >= 6) || (M == 4 && K >= 8192 && w_bits >= 6)))
+        if (fine_mode == 1 && fits_f && ((M == 1 && wide && (w_bits == 6 || w_bits == 7)) || (M == 4 && K >= 8192 && w_bits >= 6)))
             return all(AP_ROUTE_FINE);
     }
     // The 4x4x4 matrix-core kernel, whose cost per weight does not grow with M, where it measured

@@ -130,7 +130,9 @@ def test_route_report_follows_the_rule_and_the_knobs():
     from any_precision_amd import _capi
     assert _capi.matmul_route(1, 4096, 4096, 4) == "dot"
     assert _capi.matmul_route(1, 11008, 4096, 3) == "stream"
-    assert _capi.matmul_route(1, 11008, 4096, 8) == "fine"
+    assert _capi.matmul_route(1, 11008, 4096, 7) == "fine"
+    assert _capi.matmul_route(1, 11008, 4096, 8) == "dot"
+    assert _capi.matmul_geometry(1, 11008, 4096, 8)["rows"] == 1        # one row per workgroup at 8 bits
     assert _capi.matmul_route(1, 4096, 11008, 3) == "dot"
     assert _capi.matmul_route(2, 4096, 14336, 4) == "stream"
     assert _capi.matmul_route(8, 4096, 4096, 4) == "mfma16"
