@@ -33,6 +33,7 @@
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
 #include "ap_gemm_launch.hpp"
+#include "ap_lookup.hpp"
 
 namespace ap {
 
@@ -66,8 +67,12 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     constexpr int NC = 1 << BITS;
     constexpr int WPS = VEC4 ? 4 : 1;             // words per lane and step
     constexpr int ROWS = kGemmRows * RB;    // weight rows per workgroup
-    constexpr int TQ = ROWS * NC / 8;       // 16-byte quads of their tables
-    __shared__ __attribute__((aligned(16))) half_t tables[ROWS][NC];
+    // 3 and 4 bits: a table of the weights of two ADJACENT elements per row (ap_lookup.hpp) -- one ds_read_b32 per
+    // half2 of a B operand, and a quarter of the bit operations of the single-index form.
+    constexpr bool PAIR = LookupTable<BITS>::kPair;
+    constexpr int TB = LookupTable<BITS>::kBytes;  // bytes of one row's table in LDS
+    constexpr int TQ = ROWS * NC / 8;       // 16-byte quads of the rows' tables in global memory
+    __shared__ __attribute__((aligned(16))) uint8_t tables[ROWS][TB];
     // One private region per wave.  While the wave computes it stages activations there: MP rows x 16
     // octets (4 byte groups x 4 words).  Afterwards the same bytes carry the wave's partial tiles
     // (RB x MB x 4 x 64 floats) to the combine step -- LDS operations of one wave complete in order, so
@@ -121,7 +126,23 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     // array; their columns are never stored).
     uint32_t qn[RB][BITS][WPS];
     if (s_begin < s_end) fetch(s_begin, qn);
-    {
+    if constexpr (PAIR) {
+        // wave ks builds the pair tables of rows ks, ks + KS, ...: the loads of the first ROWS / 8 of them (all,
+        // when the workgroup has its eight waves) are issued together
+        constexpr int NT = ROWS / kGemmMaxSplit;
+        const PairLane<BITS> pl = pair_lane<BITS>(lane);
+        TableWords<BITS> tw[NT];
+#pragma unroll
+        for (int i = 0; i < NT; i++) {
+            const int r = min(ks + i * KS, ROWS - 1);
+            tw[i] = lookup_table_fetch<BITS>(lut + (size_t)min(n0 + r, N - 1) * NC, lane, pl);
+        }
+#pragma unroll
+        for (int i = 0; i < NT; i++)
+            if (ks + i * KS < ROWS) lookup_table_stage<BITS>(tw[i], &tables[ks + i * KS][0], lane);
+        for (int r = ks + NT * KS; r < ROWS; r += KS)
+            lookup_table_stage<BITS>(lookup_table_fetch<BITS>(lut + (size_t)min(n0 + r, N - 1) * NC, lane, pl), &tables[r][0], lane);
+    } else {
         const int nthr = KS * kWave;
         const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
         u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[0][0]);
@@ -131,7 +152,8 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     __syncthreads();
     // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
     typedef __attribute__((address_space(3))) half_t lds_half_t;
-    const uint32_t tab_base0 = (uint32_t)(uintptr_t)((lds_half_t *)&tables[0][0]) + (uint32_t)col * (NC * 2);
+    typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
+    const uint32_t tab_base0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t *)&tables[0][0]) + (uint32_t)col * TB;
 
     // byte offset of this lane's activation row in each row block (rows past M repeat row M-1)
     uint32_t xoff[MB];
@@ -224,7 +246,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
         }
         // index bytes hold the byte offset into the table (index * 2) where that fits a byte
         constexpr int PRE = BITS <= 7 ? 1 : 0;
-        uint32_t idx[RB][8];
+        uint32_t idx[RB][PAIR ? 4 : 8];
         static_for<OCT>([&](auto t_c) {
             constexpr int t = decltype(t_c)::value, wi = t / 4, j = t % 4, c = 3 - j;
             load_a(std::integral_constant<int, t + AHEAD>{});
@@ -238,29 +260,39 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
                     uint32_t qq[BITS];
 #pragma unroll
                     for (int p = 0; p < BITS; p++) qq[p] = q[rb][p][wi];
-                    planes_to_indices<BITS, PRE>(qq, idx[rb]);
+                    if constexpr (PAIR) planes_to_adjacent_pairs<BITS>(qq, idx[rb]);
+                    else planes_to_indices<BITS, PRE>(qq, idx[rb]);
                 }
             }
             // B operands: the eight weights of byte group j of each row block
             half8_t bfrag[RB];
             static_for<RB>([&](auto rb_c) {
                 constexpr int rb = decltype(rb_c)::value;
-                const uint32_t tab_base = tab_base0 + rb * (kGemmRows * NC * 2);
+                const uint32_t tab_base = tab_base0 + rb * (kGemmRows * TB);
                 u32x4 bw;
                 static_for<4>([&](auto e_c) {
                     constexpr int i = decltype(e_c)::value;
-                    uint32_t a0, a1;
-                    if constexpr (PRE) {
-                        a0 = byte_add<c>(tab_base, idx[rb][2 * i]);
-                        a1 = byte_add<c>(tab_base, idx[rb][2 * i + 1]);
+                    uint32_t packed;
+                    if constexpr (PAIR) {
+                        // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
+                        uint32_t a0;
+                        if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[rb][i]);
+                        else a0 = tab_base + byte_offset<c, 2>(idx[rb][i]);
+                        packed = *reinterpret_cast<const lds_u32_t *>(a0);
                     } else {
-                        a0 = tab_base + byte_offset<c, 1>(idx[rb][2 * i]);
-                        a1 = tab_base + byte_offset<c, 1>(idx[rb][2 * i + 1]);
+                        uint32_t a0, a1;
+                        if constexpr (PRE) {
+                            a0 = byte_add<c>(tab_base, idx[rb][2 * i]);
+                            a1 = byte_add<c>(tab_base, idx[rb][2 * i + 1]);
+                        } else {
+                            a0 = tab_base + byte_offset<c, 1>(idx[rb][2 * i]);
+                            a1 = tab_base + byte_offset<c, 1>(idx[rb][2 * i + 1]);
+                        }
+                        half2_t h;
+                        h.x = *reinterpret_cast<const lds_half_t *>(a0);
+                        h.y = *reinterpret_cast<const lds_half_t *>(a1);
+                        packed = __builtin_bit_cast(uint32_t, h);
                     }
-                    half2_t h;
-                    h.x = *reinterpret_cast<const lds_half_t *>(a0);
-                    h.y = *reinterpret_cast<const lds_half_t *>(a1);
-                    const uint32_t packed = __builtin_bit_cast(uint32_t, h);
                     bw[i] = live[wi] ? packed : 0u;
                 });
                 bfrag[rb] = __builtin_bit_cast(half8_t, bw);

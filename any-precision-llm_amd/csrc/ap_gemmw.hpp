@@ -34,10 +34,13 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemmw_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K) {
     constexpr int NC = 1 << BITS;
+    constexpr bool PAIR = LookupTable<BITS>::kPair;  // 3 and 4 bits: tables of adjacent element pairs (ap_lookup.hpp)
+    constexpr int TB = LookupTable<BITS>::kBytes;    // bytes of one row's table in LDS
     constexpr int TQ = kGemmRows * NC / 8;  // 16-byte quads of the tables of one block of rows
     constexpr int TPT = 2;                  // of which a thread carries at most two (KS >= 4)
+    constexpr int RPW = 4;                  // pair tables: rows a wave builds per block (KS >= 4)
     static_assert(MB * SPW <= 2 && TQ <= TPT * 4 * kWave, "");
-    __shared__ __attribute__((aligned(16))) half_t tables[2][kGemmRows][NC];
+    __shared__ __attribute__((aligned(16))) uint8_t tables[2][kGemmRows][TB];
     __shared__ float part[2][kGemmMaxSplit][MB * 4 * kWave];
 
     const int lane = threadIdx.x;
@@ -52,10 +55,12 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemmw_kbit_kernel(
     const uint32_t tail_stride = (uint32_t)(W & 31) * 16u;
 
     typedef __attribute__((address_space(3))) half_t lds_half_t;
+    typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
     uint32_t tab_base[2];
 #pragma unroll
     for (int b = 0; b < 2; b++)
-        tab_base[b] = (uint32_t)(uintptr_t)((lds_half_t *)&tables[b][0][0]) + (uint32_t)col * (NC * 2);
+        tab_base[b] = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t *)&tables[b][0][0]) + (uint32_t)col * TB;
+    const PairLane<BITS> pl = pair_lane<BITS>(lane);
 
     // ---- the activation operands of this wave's steps, once.  Word wi of step s is w = 16 step + 4 wi + grp;
     // its byte group j multiplies x[m][kb + j * jstride .. +7].  Words past the row end get zeros (their
@@ -100,24 +105,42 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemmw_kbit_kernel(
         }
     };
     // tables of block `blk`: contiguous in lut (rows past N re-read the last quad; their columns are never stored)
-    struct TableRegs { u32x4 v[TPT]; };
+    // pair tables: wave ks builds those of rows ks, ks + KS, ... of the block
+    struct TableRegs {
+        u32x4 v[PAIR ? 1 : TPT];
+        TableWords<BITS> w[PAIR ? RPW : 1];
+    };
     auto table_fetch = [&](int blk) {
         TableRegs r;
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
-        const long long first = (long long)blk * TQ, last = (long long)N * (NC / 8) - 1;
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int i = 0; i < TPT; i++) {
-            const int e = tid + i * nthr;
-            r.v[i] = src[min(first + min(e, TQ - 1), last)];
+            for (int i = 0; i < RPW; i++) {
+                const int row = min(blk * kGemmRows + min(ks + i * KS, kGemmRows - 1), N - 1);
+                r.w[i] = lookup_table_fetch<BITS>(lut + (size_t)row * NC, lane, pl);
+            }
+        } else {
+            const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
+            const long long first = (long long)blk * TQ, last = (long long)N * (NC / 8) - 1;
+#pragma unroll
+            for (int i = 0; i < TPT; i++) {
+                const int e = tid + i * nthr;
+                r.v[i] = src[min(first + min(e, TQ - 1), last)];
+            }
         }
         return r;
     };
     auto table_stage = [&](const TableRegs &r, int slot) {
-        u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[slot][0][0]);
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int i = 0; i < TPT; i++) {
-            const int e = tid + i * nthr;
-            if (e < TQ) dst[e] = r.v[i];
+            for (int i = 0; i < RPW; i++)
+                if (ks + i * KS < kGemmRows) lookup_table_stage<BITS>(r.w[i], &tables[slot][ks + i * KS][0], lane);
+        } else {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[slot][0][0]);
+#pragma unroll
+            for (int i = 0; i < TPT; i++) {
+                const int e = tid + i * nthr;
+                if (e < TQ) dst[e] = r.v[i];
+            }
         }
     };
 
@@ -133,31 +156,40 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemmw_kbit_kernel(
             if (ks * SPW + s < steps) {
 #pragma unroll
                 for (int p = 0; p < BITS; p++) transpose_rows4(q[s][p]);
-                uint32_t idx[8];
+                uint32_t idx[PAIR ? 4 : 8];
                 static_for<16>([&](auto t_c) {
                     constexpr int t = decltype(t_c)::value, wi = t / 4, j = t % 4, c = 3 - j;
                     if constexpr (j == 0) {
                         uint32_t qq[BITS];
 #pragma unroll
                         for (int p = 0; p < BITS; p++) qq[p] = q[s][p][wi];
-                        planes_to_indices<BITS, PRE>(qq, idx);
+                        if constexpr (PAIR) planes_to_adjacent_pairs<BITS>(qq, idx);
+                        else planes_to_indices<BITS, PRE>(qq, idx);
                     }
                     const bool live = (livemask >> (4 * s + wi)) & 1u;
                     u32x4 bw;
                     static_for<4>([&](auto e_c) {
                         constexpr int i = decltype(e_c)::value;
-                        uint32_t a0, a1;
-                        if constexpr (PRE) {
-                            a0 = byte_add<c>(tbase, idx[2 * i]);
-                            a1 = byte_add<c>(tbase, idx[2 * i + 1]);
+                        uint32_t packed;
+                        if constexpr (PAIR) {
+                            uint32_t a0;
+                            if constexpr (BITS == 3) a0 = byte_add<c>(tbase, idx[i]);
+                            else a0 = tbase + byte_offset<c, 2>(idx[i]);
+                            packed = *reinterpret_cast<const lds_u32_t *>(a0);
                         } else {
-                            a0 = tbase + byte_offset<c, 1>(idx[2 * i]);
-                            a1 = tbase + byte_offset<c, 1>(idx[2 * i + 1]);
+                            uint32_t a0, a1;
+                            if constexpr (PRE) {
+                                a0 = byte_add<c>(tbase, idx[2 * i]);
+                                a1 = byte_add<c>(tbase, idx[2 * i + 1]);
+                            } else {
+                                a0 = tbase + byte_offset<c, 1>(idx[2 * i]);
+                                a1 = tbase + byte_offset<c, 1>(idx[2 * i + 1]);
+                            }
+                            half2_t h;
+                            h.x = *reinterpret_cast<const lds_half_t *>(a0);
+                            h.y = *reinterpret_cast<const lds_half_t *>(a1);
+                            packed = __builtin_bit_cast(uint32_t, h);
                         }
-                        half2_t h;
-                        h.x = *reinterpret_cast<const lds_half_t *>(a0);
-                        h.y = *reinterpret_cast<const lds_half_t *>(a1);
-                        const uint32_t packed = __builtin_bit_cast(uint32_t, h);
                         bw[i] = live ? packed : 0u;
                     });
                     const half8_t bfrag = __builtin_bit_cast(half8_t, bw);
