@@ -352,10 +352,10 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
         const int mode = knob(kGemmWalk);
         // Where it pays (measured on 11008 / 14336 x 4096 and 28672 x 8192; 5-18 %): linears with at least 2.5
         // blocks of rows per CU to walk, at 17..32 activation rows or at 8 bits with one step per wave, and from 9
-        // rows on with two.  Elsewhere the one-shot kernels are as fast or faster (fewer rows: nothing to walk; fewer
+        // rows on with two (from 5 rows at up to 4 bits: 6-21 % on 28672 x 8192).  Elsewhere the one-shot kernels are as fast or faster (fewer rows: nothing to walk; fewer
         // activation rows at low bit-widths: their short waves hide the lookup latency better).
         const bool pays = N >= 40 * cu_count() && (gemmw_geometry(M, N, K, w_bits, &wgeo)) &&
-                          (wgeo.spw == 1 ? (M > 16 || w_bits == 8) : M > 8);
+                          (wgeo.spw == 1 ? (M > 16 || w_bits == 8) : (M > 8 || (M >= 5 && w_bits <= 4)));
         if (mode > 0 && (mode >= 2 ? gemmw_geometry(M, N, K, w_bits, &wgeo) : pays)) {
             switch (w_bits) {
                 case 3: launch_gemmw<3>(wgeo, x, qweight, lut, out, M, N, K, st); break;
@@ -378,8 +378,9 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     // 56 M weights (14336 x 4096, 8192 x 8192, 28672 x 8192: 5-25 %).
     const int rb_mode = knob(kGemmRb2);  // 0 never, 1 where it pays, 2 wherever the kernel allows
     const bool rb_fits = (W & 3) == 0 && N >= 32;
-    const bool rb_pays = M > 8 && N >= 8192 &&
-                         (w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (long long)N * K >= 56LL << 20));
+    const bool big = (long long)N * K >= 56LL << 20;
+    const bool rb_pays = N >= 8192 && (M > 8 ? (w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && big))
+                                             : (M >= 5 && w_bits == 3 && big));  // 14336 x 4096 at 5..8 rows: 6-18 %
     geo.rb = (rb_fits && (rb_mode >= 2 || (rb_mode == 1 && rb_pays))) ? 2 : 1;
     if (geo.rb == 2 && geo.mb > 2) {
         // the two-block variant exists for up to 32 activation rows: more go in chunks of 32 (the
@@ -585,8 +586,9 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     //    to 5 bits, and for 4 rows at every bit-width while a row fits one word group per lane
     //    (K <= 8192): 10-40 % faster than the dot-product kernel;
     //  - 5..8 activation rows on wide linears (16 rows per workgroup) with rows of 3072..4096 elements
-    //    (5..8 waves per workgroup): 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and longer
-    //    rows and narrower linears measured slower.
+    //    (5..8 waves per workgroup) from 4 bits on: 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and
+    //    longer rows and narrower linears measured slower, and at 3 bits the MFMA kernel with its pair-table
+    //    lookups is 4-18 % faster (11008 / 14336 x 4096).
     const int m4 = knob(kMatmulMfma4);
     long long rows = 0;
     for (int g = 0; g < count; g++) rows += N[g];
@@ -600,7 +602,7 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         }
         if (W > 16 * kGemv4MaxSegTwo) return false;
         if (m4 >= 2) return true;
-        return K >= 3072 && n >= 10240;  // per member; the others go to the MFMA kernel
+        return K >= 3072 && n >= 10240 && w_bits >= 4;  // per member; the others go to the MFMA kernel
     };
     bool any4 = false;
     for (int g = 0; g < count; g++) any4 |= use4(N[g]);

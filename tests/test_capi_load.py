@@ -137,6 +137,7 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_route(2, 4096, 14336, 4) == "stream"
     assert _capi.matmul_route(8, 4096, 4096, 4) == "mfma16"
     assert _capi.matmul_route(8, 14336, 4096, 4) == "mfma4"
+    assert _capi.matmul_route(8, 14336, 4096, 3) == "mfma16"            # pair-table lookups: faster at 3 bits
     assert _capi.matmul_route(1, 8, 32 * 64 * 2 * 17, 4) == "mfma16"      # longer than a workgroup covers
     with _capi.tuning(gemv_stream=0, gemv_fine=0):
         assert _capi.matmul_route(1, 11008, 4096, 3) == "dot"
