@@ -77,6 +77,21 @@ int check_common(int N, int K, int w_bits) {
 }
 
 // Launch geometry for `count` linears of n[0..count) rows that share K, M and w_bits.
+// Two to four activation rows on rows of at least 8192 elements (one word per lane): FOUR weight rows per workgroup,
+// so that the M x 4 KB of activations a wave loads through the L1 serve four rows.  Measured against every other
+// kernel on 4096 x 11008 / 14336, 5120 x 13824, 8192 x 8192, 28672 x 8192, 8192 x 28672 (two runs each):
+//   M = 2: 5-13 % faster than the row-streaming and two-row kernels on rows of up to 6 waves (8192, 11008
+//          elements); on longer rows mixed (-10 .. +15 %), not used;
+//   M = 3, 4: 8-40 % faster than the 4x4x4 matrix-core kernel and the two-row kernel on rows of 4 waves and of
+//          7 or more (8192, 13824, 14336, 28672 elements) at almost every bit-width -- the matrix-core kernel
+//          needs two word groups per wave there and doubles its time from 4 bits on (5120 x 13824, M = 3, 4 bits:
+//          28.9 us against 18.5) --, but 10-35 % SLOWER on rows of 11008 elements (5.4 waves), which keep their routes.
+bool long_rows_want_four(int M, int K) {
+    const int W = K >> 5, S = (W + kWave - 1) / kWave;
+    if (M < 2 || M > 4 || K < 8192 || S > kGemvMaxSeg) return false;
+    return M == 2 ? S <= 6 : (S <= 4 || S >= 7);
+}
+
 int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometry *geo, GemvMembers *mem) {
     long long rows = 0;
     for (int g = 0; g < count; g++) {
@@ -114,10 +129,11 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     if (M == 1 && wpl == 1 && force_rows <= 0 && rows * S <= 32768 &&
         (count > 1 ? w_bits >= 7 : (w_bits == 8 && K < 8192)))
         R = 1;
-    if (M == 1 && wpl == 1) {
+    if (M <= 4 && wpl == 1) {
         const long long waves = rows * S;
-        const bool pays = count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
-                                     : waves >= 20000 && w_bits <= 4;
+        const bool pays = M == 1 ? (count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
+                                               : waves >= 20000 && w_bits <= 4)
+                                 : long_rows_want_four(M, K);
         if (force_rows == 4 || (force_rows <= 0 && pays)) R = 4;
     }
     geo->wpl = wpl;
@@ -560,7 +576,8 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     //    >= 8192 elements (10-14 %);
     //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-7 bits at batch 1 on the
     //    same wide linears (3-6 %; at 8 bits gemv_kbit_kernel with one row per workgroup is faster still),
-    //    6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %).
+    //    6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %; at 6 bits on rows of up to 12288 elements the
+    //    4x4x4 kernel is 13 % faster and takes over).
     // Mode 2 of a knob forces its kernel wherever it fits (tests, sweeps); mode 0 switches it off.
     const int persist_mode = knob(kGemvPersist), fine_mode = knob(kGemvFine), stream_mode = knob(kGemvStream);
     bool fits_r = true, fits_f = true, fits_p = true;
@@ -573,11 +590,20 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     if (persist_mode >= 2 && fits_r) return all(AP_ROUTE_PERSIST);  // never the default: slower on every shape
     if (fine_mode >= 2 && fits_f) return all(AP_ROUTE_FINE);
     if (stream_mode >= 2 && fits_p) return all(AP_ROUTE_STREAM);
+    // Long rows at 2..4 activation rows: the dot-product kernel with four rows per workgroup (gemv_geometry gives
+    // it that shape) wherever long_rows_want_four says so, except that at M = 3 on rows of 7 waves or more the
+    // row-streaming kernel is 3-15 % faster still at up to 4 bits, and at M = 4 the 4x4x4 kernel keeps 3 bits
+    // (4096 x 14336, 8192 x 28672: 9 % faster than four rows).
+    const bool four = knob(kGemvRows) <= 0 && knob(kMatmulMfma4) <= 1 && geo->wpl == 1 && long_rows_want_four(M, K);
+    if (four) {
+        if (count == 1 && M == 3 && w_bits <= 4 && geo->S >= 7 && stream_mode == 1 && fits_p) return all(AP_ROUTE_STREAM);
+        if (!(M == 4 && w_bits == 3 && knob(kMatmulMfma4) == 1)) return all(AP_ROUTE_DOT);
+    }
     if (count == 1) {
         const bool wide = N[0] >= 8192 && K <= 4096;
         if (stream_mode == 1 && fits_p && ((M == 1 && wide && w_bits == 3) || (M == 2 && K >= 8192 && w_bits <= 4)))
             return all(AP_ROUTE_STREAM);
-        if (fine_mode == 1 && fits_f && ((M == 1 && wide && (w_bits == 6 || w_bits == 7)) || (M == 4 && K >= 8192 && w_bits >= 6)))
+        if (fine_mode == 1 && fits_f && ((M == 1 && wide && (w_bits == 6 || w_bits == 7)) || (M == 4 && K >= 8192 && w_bits >= (K <= 12288 ? 7 : 6))))
             return all(AP_ROUTE_FINE);
     }
     // The 4x4x4 matrix-core kernel, whose cost per weight does not grow with M, where it measured
@@ -598,7 +624,8 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         if (M <= 4) {  // decided for the group as a whole, by its mean row count
             if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
             if (m4 >= 2) return true;
-            return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192))) && rows >= 2048LL * count;
+            return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192 || (w_bits == 6 && K <= 12288)))) &&
+                   rows >= 2048LL * count;
         }
         if (W > 16 * kGemv4MaxSegTwo) return false;
         if (m4 >= 2) return true;

@@ -30,7 +30,7 @@ void launch_m(const GemvGeometry &geo, const half_t *x, const GemvMembers &mem, 
         }
         if (geo.R == 1) return launch_rows<BITS, M, 1, 1>(geo, x, mem, K, stream);
     }
-    if constexpr (M == 1) {  // four rows per workgroup exist for one activation row only
+    if constexpr (M <= 4) {  // four rows per workgroup exist for up to four activation rows
         if (geo.R == 4) return launch_rows<BITS, M, 1, 4>(geo, x, mem, K, stream);
     }
     launch_rows<BITS, M, 1, 2>(geo, x, mem, K, stream);

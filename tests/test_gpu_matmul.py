@@ -376,17 +376,24 @@ def test_four_rows_per_workgroup_agree_with_the_oracle(ext, oracle):
         L = make(N, K, seed=N + K)
         q, luts = layer_to_gpu(L)
         for b in range(3, 9):
-            print(f"four rows N={N} K={K} b={b}", flush=True)
-            x, xg = _x(1, K, seed=b)
-            with _capi.tuning(gemv_rows=4, gemv_stream=0, gemv_fine=0):
-                assert _capi.matmul_geometry(1, N, K, b)["rows"] == 4
-                got = ext.matmul_kbit(xg, q, luts[b], b)
-            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
-            assert_close_gemv(got, want, f"N={N} K={K} b={b}")
+            for M in (1, 2, 3, 4):
+                print(f"four rows N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=b + M)
+                with _capi.tuning(gemv_rows=4, gemv_stream=0, gemv_fine=0, matmul_mfma4=0):
+                    assert _capi.matmul_geometry(M, N, K, b)["rows"] == 4 and _capi.matmul_route(M, N, K, b) == "dot"
+                    got = ext.matmul_kbit(xg, q, luts[b], b)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                assert_close_gemv(got, want, f"N={N} K={K} b={b} M={M}")
     assert _capi.matmul_geometry(1, 14336, 4096, 3)["rows"] == 4      # 28672 waves at 3 bits
     assert _capi.matmul_geometry(1, 14336, 4096, 6)["rows"] == 2
     assert _capi.matmul_geometry(1, 14336, 4096, 8)["rows"] == 1      # one row at 8 bits on short rows
     assert _capi.matmul_geometry(1, 8192, 8192, 8)["rows"] == 4       # long rows: at every bit-width
     assert _capi.matmul_geometry(1, 4096, 11008, 3)["rows"] == 2
     assert _capi.matmul_geometry(1, 4096, 4096, 3)["rows"] == 1
-    assert _capi.matmul_geometry(2, 14336, 4096, 3)["rows"] == 2      # one activation row only
+    assert _capi.matmul_geometry(2, 14336, 4096, 3)["rows"] == 2      # short rows: four only at one activation row
+    # 2..4 activation rows on long rows: four rows per workgroup, except rows of 5..6 waves at M = 3, 4 and of 7+ at M = 2
+    for M, N, K, rows, route in ((2, 4096, 11008, 4, "dot"), (2, 4096, 14336, 2, "stream"), (3, 4096, 14336, 4, "stream"),
+                                 (3, 8192, 8192, 4, "dot"), (3, 4096, 11008, 2, "mfma4"), (4, 5120, 13824, 4, "dot"),
+                                 (4, 28672, 8192, 4, "dot")):
+        assert _capi.matmul_geometry(M, N, K, 4)["rows"] == rows and _capi.matmul_route(M, N, K, 4) == route, (M, N, K)
+    assert _capi.matmul_route(4, 4096, 14336, 3) == "mfma4" and _capi.matmul_route(3, 5120, 13824, 6) == "dot"
