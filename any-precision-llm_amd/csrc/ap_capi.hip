@@ -115,9 +115,10 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // One row per workgroup until that would launch more than target_waves waves, then two
     // (the second row reuses the activation registers; more rows lengthen the compute
     // tail).  From M = 3 on the activations are the larger load: always two rows.
-    // At 3-4 bits (least work per wave) the switch comes at three quarters of that: 5120 x 5120 (15360 waves) is
-    // 8-15 % faster with two rows there, within 3 % either way from 5 bits on; 4096 x 4096 (8192 waves) keeps one.
-    const long long tw = target_waves > 0 ? (w_bits <= 4 ? (long long)target_waves * 3 / 4 : target_waves) : 1;
+    // At 3-4 bits (least work per wave) and at two activation rows the switch comes at three quarters of that:
+    // 5120 x 5120 (15360 waves) is 8-15 % faster with two rows there (M = 1: within 3 % either way from 5 bits
+    // on); 4096 x 4096 (8192 waves) keeps one.
+    const long long tw = target_waves > 0 ? ((w_bits <= 4 || M == 2) ? (long long)target_waves * 3 / 4 : target_waves) : 1;
     int R = force_rows > 0 ? force_rows : (int)((rows * S + tw - 1) / (tw > 0 ? tw : 1));
     R = (R >= 2 || M > 2) ? 2 : 1;
     // Four rows per workgroup (one activation row, one word per lane): the activations a wave holds then serve
