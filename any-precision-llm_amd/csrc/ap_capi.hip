@@ -115,17 +115,20 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // One row per workgroup until that would launch more than target_waves waves, then two
     // (the second row reuses the activation registers; more rows lengthen the compute
     // tail).  From M = 3 on the activations are the larger load: always two rows.
-    // At 3-4 bits (least work per wave) and at two activation rows the switch comes at three quarters of that:
+    // At 3-4 bits (least work per wave) and for a single linear at two activation rows the switch comes at three quarters of that:
     // 5120 x 5120 (15360 waves) is 8-15 % faster with two rows there (M = 1: within 3 % either way from 5 bits
     // on); 4096 x 4096 (8192 waves) keeps one.
-    const long long tw = target_waves > 0 ? ((w_bits <= 4 || M == 2) ? (long long)target_waves * 3 / 4 : target_waves) : 1;
-    int R = force_rows > 0 ? force_rows : (int)((rows * S + tw - 1) / (tw > 0 ? tw : 1));
+    const long long tw = target_waves > 0 ? ((w_bits <= 4 || (M == 2 && count == 1)) ? (long long)target_waves * 3 / 4 : target_waves) : 1;
+    int R = force_rows > 0 ? force_rows : (rows * S >= tw ? 2 : 1);
     R = (R >= 2 || M > 2) ? 2 : 1;
     // Four rows per workgroup (one activation row, one word per lane): the activations a wave holds then serve
     // four rows, which halves their traffic through the L1 once more, at the price of half the waves.  Measured
     // 3-6 % faster (two boxes, run-to-run noise about as large) on single linears of at least 28000 waves at up to
     // 4 bits (14336 x 4096, 4096 x 14336) and, with rows of at least 8192 elements, at every bit-width
     // (8192 x 8192, 28672 x 8192); equal or slower on the Llama-2-7B shapes, so those keep two.
+    // Launches of several linears at 2..4 activation rows (q/k/v, gate/up of the 7B / 8B / 13B / 70B models, swept at
+    // 3, 4, 5, 8 bits): four rows at M = 3, 4 at every bit-width (the one launch is 20-46 % faster than a 4x4x4
+    // launch per member and 5-20 % faster than two rows), and at M = 2 at up to 4 bits (4-12 %; 3-9 % slower at 5 bits).
     // At the highest bit-widths the lookups want more waves in flight: ONE row per workgroup up to 32768 waves is
     // 8-15 % faster at 7-8 bits for launches of several linears (q/k/v: 3 x 4096 x 4096 = 24576 waves) and 2-7 %
     // faster at 8 bits for single wide ones of short rows (11008 / 14336 x 4096).  At 3-4 bits launches of several
@@ -137,7 +140,7 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
         const long long waves = rows * S;
         const bool pays = M == 1 ? (count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
                                                : waves >= 20000 && w_bits <= 4)
-                                 : long_rows_want_four(M, K);
+                                 : long_rows_want_four(M, K) || (count > 1 && (M >= 3 || w_bits <= 4));
         if (force_rows == 4 || (force_rows <= 0 && pays)) R = 4;
     }
     geo->wpl = wpl;
@@ -628,6 +631,7 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         if (M <= 4) {  // decided for the group as a whole, by its mean row count
             if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
             if (m4 >= 2) return true;
+            if (count > 1) return false;  // several linears: one dot-product launch with four rows per workgroup beats a launch each
             return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192 || (w_bits == 6 && K <= 12288)))) &&
                    rows >= 2048LL * count;
         }
