@@ -625,6 +625,31 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     const int m4 = knob(kMatmulMfma4);
     long long rows = 0;
     for (int g = 0; g < count; g++) rows += N[g];
+    // 5..8 activation rows where the dot-product kernel (cost linear in M, one launch for all members) still beats
+    // the matrix-core kernels (cost flat in M, one launch per member, 16 rows per workgroup).  Swept at M = 5..8,
+    // 3..8 bits, on the 7B / 8B / 13B / 70B linears and their q/k/v and gate/up sets (default knobs only):
+    //  - a linear of at most 2048 rows (k/v projections with grouped heads: 64-128 workgroups of the MFMA kernel):
+    //    10-54 % faster at every M and bit-width; a set with such a member 6-50 % (at M >= 7 on rows of more than
+    //    4096 elements only from 5 bits on);
+    //  - 7-8 bits on linears of >= 5120 rows of 4097..8192 elements, where the MFMA kernel is at its worst (5120 x
+    //    5120, 13824 x 5120, 8192 x 8192, 28672 x 8192): 10-41 % at M = 5, 6 at 8 bits and 9-20 % at M = 5 at 7 bits;
+    //  - sets at M = 5: 8-46 % at 8 bits, and 15-37 % from 5 bits on when no member has more than 8192 rows.
+    auto dot_beats_mfma = [&]() {
+        if (M < 5 || M > 8 || knob(kMatmulMfmaFrom) != 5 || m4 >= 2 || geo->wpl != 1) return false;
+        int lo = N[0], hi = N[0];
+        for (int g = 1; g < count; g++) {
+            lo = N[g] < lo ? N[g] : lo;
+            hi = N[g] > hi ? N[g] : hi;
+        }
+        if (count == 1) {
+            if (lo <= 2048) return true;
+            return K > 4096 && K <= 8192 && lo >= 5120 && ((w_bits == 8 && M <= 6) || (w_bits == 7 && M == 5));
+        }
+        if (lo <= 2048 && (M <= 6 || K <= 4096 || w_bits >= 5)) return true;
+        if (w_bits == 8 && K > 4096 && K <= 8192) return true;  // every M: 3-32 % (13B / 70B sets)
+        return M == 5 && (w_bits == 8 || (w_bits >= 5 && hi <= 8192));
+    };
+    if (dot_beats_mfma()) return all(AP_ROUTE_DOT);
     auto use4 = [&](int n) {
         const int W = K >> 5;
         if (m4 == 0 || M < 2 || M > 8) return false;
