@@ -377,7 +377,9 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
         // blocks of rows per CU to walk, at 17..32 activation rows or at 8 bits with one step per wave, and from 9
         // rows on with two (from 5 rows at up to 4 bits: 6-21 % on 28672 x 8192).  Elsewhere the one-shot kernels are as fast or faster (fewer rows: nothing to walk; fewer
         // activation rows at low bit-widths: their short waves hide the lookup latency better).
-        const bool pays = N >= 40 * cu_count() && (gemmw_geometry(M, N, K, w_bits, &wgeo)) &&
+        // With two steps per wave it needs twice the rows (28672 x 8192: 5-21 %; on 13824 x 5120 the two-block
+        // one-shot kernel is up to 20 % faster).
+        const bool pays = gemmw_geometry(M, N, K, w_bits, &wgeo) && N >= 40 * wgeo.spw * cu_count() &&
                           (wgeo.spw == 1 ? (M > 16 || w_bits == 8) : (M > 8 || (M >= 5 && w_bits <= 4)));
         if (mode > 0 && (mode >= 2 ? gemmw_geometry(M, N, K, w_bits, &wgeo) : pays)) {
             switch (w_bits) {
@@ -401,9 +403,13 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     // 56 M weights (14336 x 4096, 8192 x 8192, 28672 x 8192: 5-25 %).
     const int rb_mode = knob(kGemmRb2);  // 0 never, 1 where it pays, 2 wherever the kernel allows
     const bool rb_fits = (W & 3) == 0 && N >= 32;
+    // Linears of 5120..8191 rows (5120 x 5120, 5120 x 13824; swept later) gain as much: 19-38 % at 3 bits, 3-22 % at
+    // 5 bits; and at 8 bits up to 16 activation rows gain 8-16 % wherever a wave has more than one step (rows of
+    // more than 4096 elements: 5120 x 5120, 13824 x 5120, 5120 x 13824, 8192 x 8192, 8192 x 28672).
     const bool big = (long long)N * K >= 56LL << 20;
-    const bool rb_pays = N >= 8192 && (M > 8 ? (w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && big))
-                                             : (M >= 5 && w_bits == 3 && big));  // 14336 x 4096 at 5..8 rows: 6-18 %
+    const bool low_bits = w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (big || N < 8192));
+    const bool rb_pays = N >= 5120 && (M > 8 ? (low_bits || (w_bits == 8 && M <= 16 && K > 4096))
+                                             : (M >= 5 && w_bits == 3 && big && N >= 8192));  // 14336 x 4096 at 5..8 rows: 6-18 %
     geo.rb = (rb_fits && (rb_mode >= 2 || (rb_mode == 1 && rb_pays))) ? 2 : 1;
     if (geo.rb == 2 && geo.mb > 2) {
         // the two-block variant exists for up to 32 activation rows: more go in chunks of 32 (the
