@@ -92,6 +92,10 @@ bool long_rows_want_four(int M, int K) {
     return M == 2 ? S <= 6 : (S <= 4 || S >= 7);
 }
 
+// Four activation rows at 6-8 bits on rows of 4097..8191 elements (5120 x 5120, 13824 x 5120): four weight rows per
+// workgroup too, 9-13 % faster than the 4x4x4 kernel there (equal or slower at fewer bits and at three rows).
+bool mid_rows_want_four(int M, int K, int w_bits) { return M == 4 && w_bits >= 6 && K > 4096 && K < 8192; }
+
 int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometry *geo, GemvMembers *mem) {
     long long rows = 0;
     for (int g = 0; g < count; g++) {
@@ -140,7 +144,8 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
         const long long waves = rows * S;
         const bool pays = M == 1 ? (count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
                                                : waves >= 20000 && w_bits <= 4)
-                                 : long_rows_want_four(M, K) || (count > 1 && (M >= 3 || w_bits <= 4));
+                                 : long_rows_want_four(M, K) || mid_rows_want_four(M, K, w_bits) ||
+                                   (count > 1 && (M >= 3 || w_bits <= 4));
         if (force_rows == 4 || (force_rows <= 0 && pays)) R = 4;
     }
     geo->wpl = wpl;
@@ -409,7 +414,8 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     const bool big = (long long)N * K >= 56LL << 20;
     const bool low_bits = w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (big || N < 8192));
     const bool rb_pays = N >= 5120 && (M > 8 ? (low_bits || (w_bits == 8 && M <= 16 && K > 4096))
-                                             : (M >= 5 && w_bits == 3 && big && N >= 8192));  // 14336 x 4096 at 5..8 rows: 6-18 %
+                                             : (M >= 5 && ((w_bits == 3 && big && N >= 8192) ||  // 14336 x 4096 at 5..8 rows: 6-18 %
+                                                           (K >= 8192 && N <= 8192))));  // 5120 x 13824, 8192 x 28672, 8192 x 8192: 5-17 %
     geo.rb = (rb_fits && (rb_mode >= 2 || (rb_mode == 1 && rb_pays))) ? 2 : 1;
     if (geo.rb == 2 && geo.mb > 2) {
         // the two-block variant exists for up to 32 activation rows: more go in chunks of 32 (the
@@ -608,6 +614,11 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     // row-streaming kernel is 3-15 % faster still at up to 4 bits, and at M = 4 the 4x4x4 kernel keeps 3 bits
     // (4096 x 14336, 8192 x 28672: 9 % faster than four rows).
     const bool four = knob(kGemvRows) <= 0 && knob(kMatmulMfma4) <= 1 && geo->wpl == 1 && long_rows_want_four(M, K);
+    // narrow linears (k/v projections with grouped heads) at 2..4 rows: the fine-grained kernel, 5-15 % on 1024 x 8192,
+    // 5-9 % on 1024 x 4096 at 3-4 rows and up to 4 bits
+    if (count == 1 && fine_mode == 1 && fits_f && N[0] <= 2048 &&
+        ((K >= 8192 && M >= 2 && M <= 4) || (M >= 3 && M <= 4 && w_bits <= 4)))
+        return all(AP_ROUTE_FINE);
     if (four) {
         if (count == 1 && M == 3 && w_bits <= 4 && geo->S >= 7 && stream_mode == 1 && fits_p) return all(AP_ROUTE_STREAM);
         if (!(M == 4 && w_bits == 3 && knob(kMatmulMfma4) == 1)) return all(AP_ROUTE_DOT);
@@ -637,8 +648,9 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     //  - a linear of at most 2048 rows (k/v projections with grouped heads: 64-128 workgroups of the MFMA kernel):
     //    10-54 % faster at every M and bit-width; a set with such a member 6-50 % (at M >= 7 on rows of more than
     //    4096 elements only from 5 bits on);
-    //  - 7-8 bits on linears of >= 5120 rows of 4097..8192 elements, where the MFMA kernel is at its worst (5120 x
-    //    5120, 13824 x 5120, 8192 x 8192, 28672 x 8192): 10-41 % at M = 5, 6 at 8 bits and 9-20 % at M = 5 at 7 bits;
+    //  - 7-8 bits on linears of >= 5120 rows of more than 4096 elements, where the MFMA kernel is at its worst (5120 x
+    //    5120, 13824 x 5120, 8192 x 8192, 28672 x 8192): 7-41 % at M = 5..7 at 8 bits (M = 8 too on rows of 5120
+    //    elements; M = 5 only on rows of 8193..16384: 5120 x 13824, 22 %; never beyond) and 9-20 % at M = 5 at 7 bits;
     //  - sets at M = 5: 8-46 % at 8 bits, and 15-37 % from 5 bits on when no member has more than 8192 rows.
     auto dot_beats_mfma = [&]() {
         if (M < 5 || M > 8 || knob(kMatmulMfmaFrom) != 5 || m4 >= 2 || geo->wpl != 1) return false;
@@ -649,7 +661,10 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         }
         if (count == 1) {
             if (lo <= 2048) return true;
-            return K > 4096 && K <= 8192 && lo >= 5120 && ((w_bits == 8 && M <= 6) || (w_bits == 7 && M == 5));
+            if (K <= 4096 || lo < 5120) return false;
+            if (w_bits == 8) return K <= 8192 ? (M <= 7 || K <= 5120) : (M == 5 && K <= 16384);
+            if (w_bits == 7) return M == 5 && K <= 8192;
+            return M == 5 && w_bits >= 5 && (long long)lo * K <= 32LL << 20;  // 5120 x 5120: 14-16 %
         }
         if (lo <= 2048 && (M <= 6 || K <= 4096 || w_bits >= 5)) return true;
         if (w_bits == 8 && K > 4096 && K <= 8192) return true;  // every M: 3-32 % (13B / 70B sets)
@@ -663,6 +678,7 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
             if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
             if (m4 >= 2) return true;
             if (count > 1) return false;  // several linears: one dot-product launch with four rows per workgroup beats a launch each
+            if (mid_rows_want_four(M, K, w_bits)) return false;
             return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192 || (w_bits == 6 && K <= 12288)))) &&
                    rows >= 2048LL * count;
         }

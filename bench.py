@@ -34,7 +34,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--workload", default="llama2_7b_layer_batch1",
                     choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model",
-                             "llama2_7b_decode", "llama2_7b_prefill", "gemv_kernel_variants"),
+                             "llama2_7b_decode", "llama2_7b_prefill", "gemv_kernel_variants", "routing_audit"),
                     help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
                          "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
                          "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.  "
@@ -44,7 +44,12 @@ def parse_args():
                          "(dequant_kbit + library GEMM, the large-batch branch of AnyPrecisionLinear).  "
                          "gemv_kernel_variants: the four dot-product GEMV kernels forced in turn (tuning knobs) on "
                          "the headline shapes and on 28672 x 8192, batch 1, beside the read-only stream; with "
-                         "--eager the launches go out one by one (the form rocprofv3 counter runs need).")
+                         "--eager the launches go out one by one (the form rocprofv3 counter runs need).  "
+                         "routing_audit: for the linears of the models named by --audit-models, at 1..8 activation "
+                         "rows and 3, 4, 5, 8 bits, the time of what ap_matmul_kbit launches by default beside every "
+                         "kernel and geometry the tuning knobs can force: where is the default not the fastest.")
+    ap.add_argument("--audit-models", default="7b,8b", help="routing_audit: comma list out of 7b, 8b, 13b, 70b")
+    ap.add_argument("--audit-rows", default="1,2,3,4,5,8", help="routing_audit: activation row counts")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -100,6 +105,8 @@ def main():
         return prefill_linears(args, torch, _capi, synth)
     if args.workload == "gemv_kernel_variants":
         return gemv_kernel_variants(args, torch, _capi, synth)
+    if args.workload == "routing_audit":
+        return routing_audit(args, torch, _capi, synth)
     if args.workload == "llama2_7b_decode":
         with torch.inference_mode():     # the decoder captures its graphs in inference mode; stay in it
             return decode_tokens(args, torch, _capi, synth)
@@ -699,6 +706,82 @@ def gemv_kernel_variants(args, torch, _capi, synth):
                                "dot / fine / stream / persist kernels forced through ap_set_tuning; cold weight sets; "
                                + ("eager launches" if args.eager else "HIP graphs")},
         "value": None, "kernels": rows}))
+
+
+AUDIT_SHAPES = {   # (rows, elements per row) of the distinct linears of a decoder layer
+    "7b": ((4096, 4096), (11008, 4096), (4096, 11008)),
+    "8b": ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)),
+    "13b": ((5120, 5120), (13824, 5120), (5120, 13824)),
+    "70b": ((8192, 8192), (1024, 8192), (28672, 8192), (8192, 28672)),
+}
+
+
+def routing_audit(args, torch, _capi, synth):
+    """ap_matmul_kbit's own choice of kernel and launch geometry against every alternative the tuning knobs can
+    force, on cold weight sets: per (shape, activation rows, w_bits) the default's time, the fastest candidate's,
+    and which it was.  The routing rules are thresholds fitted to measurements; this is the measurement."""
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    side = torch.cuda.Stream()
+    bits = (3, 4, 5, 8)
+    dot = {"gemv_stream": 0, "gemv_fine": 0, "matmul_mfma4": 0}
+    few = [("dot_1row", dict(dot, gemv_rows=1)), ("dot_2rows", dict(dot, gemv_rows=2)), ("dot_4rows", dict(dot, gemv_rows=4)),
+           ("stream", {"gemv_stream": 2}), ("fine", {"gemv_fine": 2}), ("mfma4", {"matmul_mfma4": 2, "gemv_stream": 0, "gemv_fine": 0})]
+    many = [("dot", dict(dot, matmul_mfma_from=9)), ("mfma16", {"matmul_mfma4": 0, "matmul_mfma_from": 4}),
+            ("mfma16_2blocks", {"matmul_mfma4": 0, "matmul_mfma_from": 4, "gemm_rb2": 2, "gemm_walk": 0}),
+            ("mfma4", {"matmul_mfma4": 2})]
+    shapes = []
+    for m in args.audit_models.split(","):
+        for sh in AUDIT_SHAPES[m.strip()]:
+            if sh not in shapes:
+                shapes.append(sh)
+    Ms = [int(v) for v in args.audit_rows.split(",")]
+    cases, losses = [], []
+    for N, K in shapes:
+        sets = max(4, int(args.pool_gb * 1e9 / (N * K)) + 1)
+        P = WeightPool(torch, N, K, sets, gen, bits=bits)
+        cur = {"j": 0}
+        for b in bits:
+            for M in Ms:
+                x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+
+                def gemv(st):
+                    cur["j"] = (cur["j"] + 1) % P.sets
+                    rc = lib.ap_matmul_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                            P.out.data_ptr(), M, N, K, b, st)
+                    if rc != 0:
+                        raise RuntimeError(_capi.strerror(rc))
+
+                reps = min(P.sets, 24)
+                us = {"default": _graph_us(torch, side, gemv, reps)}
+                for name, knobs in (few if M <= 4 else many):
+                    if name == "mfma4" and M < 2:
+                        continue
+                    with _capi.tuning(**knobs):
+                        if _capi.matmul_route(M, N, K, b) != name.split("_")[0]:
+                            continue                      # the kernel does not serve this shape
+                        if name.startswith("dot_") and _capi.matmul_geometry(M, N, K, b)["rows"] != int(name[4]):
+                            continue                      # nor with this many rows per workgroup
+                        us[name] = _graph_us(torch, side, gemv, reps)
+                us["default"] = min(us["default"], _graph_us(torch, side, gemv, reps))   # measured first and last
+                best = min((k for k in us if k != "default"), key=lambda k: us[k], default="default")
+                case = {"N": N, "K": K, "w_bits": b, "M": M, "route": _capi.matmul_route(M, N, K, b),
+                        "default_us": round(us["default"], 2), "best": best, "best_us": round(us[best], 2)}
+                cases.append(case)
+                if us["default"] > 1.05 * us[best]:
+                    losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
+        del P
+        torch.cuda.empty_cache()
+    within = 1 - len(losses) / len(cases)
+    print(json.dumps({
+        "metric": "share of (shape, rows, w_bits) cases where ap_matmul_kbit's default launch is within 5 % of the fastest forced alternative",
+        "value": round(within, 4), "unit": "fraction", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None,
+        "data": "synthetic", "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate",
+        "config": {"workload": f"linears of {args.audit_models} at {args.audit_rows} activation rows, w_bits 3, 4, 5, 8; cold weight "
+                               "sets; HIP graphs; alternatives forced through ap_set_tuning"},
+        "cases": len(cases), "worst_excess": max((l["excess"] for l in losses), default=0.0),
+        "losses": sorted(losses, key=lambda l: -l["excess"]), "all_cases": cases}))
 
 
 def dequant_full_model(args, torch, _capi, synth):

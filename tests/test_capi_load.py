@@ -139,7 +139,8 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_route(8, 14336, 4096, 4) == "mfma4"
     assert _capi.matmul_route(8, 14336, 4096, 3) == "mfma16"            # pair-table lookups: faster at 3 bits
     assert _capi.matmul_route(8, 1024, 4096, 3) == "dot"                # too few rows for 16 per workgroup
-    assert _capi.matmul_route(5, 5120, 5120, 8) == "dot" and _capi.matmul_route(8, 5120, 5120, 8) == "mfma16"
+    assert _capi.matmul_route(5, 5120, 5120, 8) == "dot" and _capi.matmul_route(8, 8192, 8192, 8) == "mfma16"
+    assert _capi.matmul_route(5, 8192, 28672, 8) == "mfma16" and _capi.matmul_route(3, 1024, 8192, 5) == "fine"
     with _capi.tuning(matmul_mfma_from=5, matmul_mfma4=2):
         assert _capi.matmul_route(8, 1024, 4096, 3) != "dot"            # a forced kernel overrides the rule
     assert _capi.matmul_route(1, 8, 32 * 64 * 2 * 17, 4) == "mfma16"      # longer than a workgroup covers
