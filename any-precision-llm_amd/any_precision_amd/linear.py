@@ -20,14 +20,18 @@ except ModuleNotFoundError:
 
 
 def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int = 0) -> bool:
-    """Whether the fused GEMM beats dequant_kbit + torch.matmul (measured on the Llama-2-7B / Llama-3-8B
-    / 8192 x 8192 shapes, every bit-width): always up to 32 activation rows (1.3-2.6x at 16); up to 64
-    on linears of fewer than 8192 rows, and on larger ones at up to 5 bits; up to 128 on linears of fewer
-    than 8192 rows of at most 4096 elements (4096 x 4096: 33-35 us against 43).  Beyond, the re-read of
-    the activations per block of weight rows costs more than materialising the weight once."""
+    """Whether the fused GEMM beats dequant_kbit + torch.matmul (measured on the 13 distinct linears of the
+    Llama-2-7B / Llama-3-8B / 13B / 70B layers at 3, 5, 8 bits): always up to 32 activation rows (1.3-4x at 16);
+    up to 64 on linears of fewer than 8192 rows, and on larger ones at up to 5 bits -- except, on rows of more
+    than 4096 elements, from 6 bits on linears of 5120 rows or more (5120 x 13824, 8 bits: 121 us against 86)
+    and from 5 bits on linears of at most 2048 rows (1024 x 8192); up to 128 on linears of fewer than 8192
+    rows of at most 4096 elements (4096 x 4096: 33-35 us against 43).  Beyond, the re-read of the
+    activations per block of weight rows costs more than materialising the weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
     if rows <= min(64, GEMM_MAX_M):
+        if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):
+            return False
         return out_features < 8192 or w_bits <= 5
     return rows <= min(128, GEMM_MAX_M) and out_features < 8192 and 0 < in_features <= 4096
 

@@ -57,3 +57,5 @@ def test_fused_gemm_dispatch_rule():
     assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6)
     assert not fused_gemm_pays(65, 4096, 3) and not fused_gemm_pays(65, 4096, 3, 11008) and not fused_gemm_pays(129, 4096, 3, 4096)
     assert fused_gemm_pays(128, 4096, 8, 4096) and not fused_gemm_pays(128, 11008, 3, 4096)
+    assert fused_gemm_pays(64, 5120, 5, 13824) and not fused_gemm_pays(64, 5120, 8, 13824)      # long rows, 6 bits on
+    assert fused_gemm_pays(64, 1024, 8, 4096) and not fused_gemm_pays(64, 1024, 5, 8192)        # narrow, long rows
