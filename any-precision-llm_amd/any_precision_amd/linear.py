@@ -39,13 +39,14 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
 def forward_group(modules, x, precision=None, concat=False):
     """``[m(x, precision=precision) for m in modules]`` for linears that share their input (the
     q/k/v or gate/up projections of a decoder layer); with ``concat`` the results joined along
-    the last dimension.  Up to 4 activation rows and 4 modules the GEMVs go out as ONE launch;
-    otherwise module by module.  The reference has no counterpart (its ``fuse_layers`` is a
+    the last dimension.  Up to 8 activation rows and 4 modules they go through ``matmul_kbit_group``, which
+    issues ONE launch wherever the dot-product kernel serves the set (always up to 4 rows; at 5..8 rows for
+    sets with narrow members and some 5-8-bit cases) and a launch per member otherwise; beyond, module by module.  The reference has no counterpart (its ``fuse_layers`` is a
     stub, AnyPrecisionForCausalLM.py:168-172)."""
     rows = x.numel() // x.shape[-1]
     w_bits = modules[0].precision if precision is None else precision
     x = x.contiguous()
-    if rows > 4 or not 2 <= len(modules) <= 4 or any(
+    if rows > 8 or not 2 <= len(modules) <= 4 or any(
             m.in_features != modules[0].in_features for m in modules):
         outs = [m(x, precision=w_bits) for m in modules]
         return torch.cat(outs, dim=-1) if concat else outs

@@ -82,3 +82,33 @@ def test_constructor_errors():
         AnyPrecisionLinear(64, 8, [3, 4], dtype=torch.float32)
     with pytest.raises(RuntimeError):
         AnyPrecisionLinear(64, 8, [3, 4], precisions=(3, 4))
+
+
+def test_forward_group_equals_module_by_module(oracle):
+    """forward_group (one launch where the dot-product kernel serves the set, a launch per member otherwise, module
+    by module beyond 8 rows) against the modules called one by one: the oracle's values at the path's bar, with
+    and without biases, joined or as a list."""
+    from any_precision_amd.linear import forward_group, forward_swiglu
+    layers = [make(n, 4096, seed=70 + n) for n in (256, 64, 64)]
+    for bias in (False, True):
+        mods = [_module(L, bias=bias)[0] for L in layers]
+        for b in (3, 8):
+            for rows in (1, 3, 6, 8, 9):
+                print(f"forward_group bias={bias} b={b} rows={rows}", flush=True)
+                x = synth.make_x(rows, 4096, seed=rows)
+                xg = torch.from_numpy(x).cuda()
+                outs = forward_group(mods, xg, b)
+                joined = forward_group(mods, xg, b, concat=True)
+                assert joined.shape == (rows, 384) and torch.equal(joined, torch.cat(outs, dim=-1))
+                for L, m, got in zip(layers, mods, outs):
+                    _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                    if bias:
+                        want = want + m.bias.double().cpu().numpy()
+                    assert_close_gemv(got, want, f"forward_group bias={bias} b={b} rows={rows} N={L.N}")
+    # SiLU(gate) * up through the one-launch form (up to 4 rows) and through its fallback
+    gate, up = _module(layers[1], bias=False)[0], _module(layers[2], bias=False)[0]
+    for rows in (2, 6):
+        xg = torch.from_numpy(synth.make_x(rows, 4096, seed=9)).cuda()
+        got = forward_swiglu(gate, up, xg, 4)
+        want = torch.nn.functional.silu(gate(xg, precision=4).float()) * up(xg, precision=4).float()
+        assert (got.float() - want).abs().max().item() <= 1e-2 * want.abs().max().item()
