@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libanyprec_hip.so")
 
 AP_OK = 0
 AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT, AP_EKNOB = -1, -2, -3, -4, -5, -6, -7
-AP_ABI_VERSION = 5
+AP_ABI_VERSION = 6
 
 if not os.path.exists(LIB_PATH):
     raise ModuleNotFoundError(
@@ -55,6 +55,8 @@ lib.ap_silu_mul.argtypes = [_vp, _vp, _vp, ctypes.c_longlong, _vp]
 lib.ap_silu_mul.restype = _ci
 lib.ap_decode_attention.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, ctypes.c_float, _vp]
 lib.ap_decode_attention.restype = _ci
+lib.ap_decode_advance.argtypes = [_vp, _ci, _vp, _vp, _vp, _ci, _vp]
+lib.ap_decode_advance.restype = _ci
 lib.ap_set_tuning.argtypes = [ctypes.c_char_p, _ci]
 lib.ap_set_tuning.restype = _ci
 lib.ap_get_tuning.argtypes = [ctypes.c_char_p, _pi]
@@ -67,7 +69,7 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
            "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_probe_write", "ap_matmul_kbit_route",
-           "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu")
+           "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu", "ap_decode_advance")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
 

@@ -23,6 +23,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _capi
+from .decode_ops import advance
 from .linear import forward_group, forward_swiglu
 
 
@@ -158,7 +159,7 @@ class GraphDecoder:
             _capi.check(lib.ap_add_rmsnorm(self.f_h.data_ptr(), 0 if delta is None else delta.data_ptr(), weight.data_ptr(),
                                            self.f_h.data_ptr(), self.f_x.data_ptr(), 1, H, eps, st), "ap_add_rmsnorm")
 
-        self.f_h.copy_(self.embed.index_select(0, self.tok))
+        torch.index_select(self.embed, 0, self.tok, out=self.f_h)
         delta = None
         for li, layer in enumerate(self.layers):
             att = layer.self_attn
@@ -179,14 +180,15 @@ class GraphDecoder:
                 _capi.check(lib.ap_silu_mul(gate.data_ptr(), up.data_ptr(), self.f_act.data_ptr(), gate.numel(), st), "ap_silu_mul")
             delta = layer.mlp.down_proj(self.f_act, precision=precision)
         add_norm(delta, self.final_norm)
-        return F.linear(self.f_x, self.head)
+        return torch.mm(self.f_x, self.head.t(), out=self.logits)
 
     def _step(self, precision):
         """One decode step on the static state: consumes self.tok at self.pos, leaves the next token."""
         if self.fused_ops:
-            logits = self._forward_fused(precision)
-        else:
-            logits = self._forward(self.tok, self.pos, precision)
+            self._forward_fused(precision)           # writes self.logits
+            advance(self.logits, self.pos, self.tok, self.emitted)
+            return
+        logits = self._forward(self.tok, self.pos, precision)
         self.logits.copy_(logits)
         nxt = torch.argmax(logits, dim=-1)
         self.pos.add_(1)

@@ -1,5 +1,5 @@
 """Tensor-level wrappers of the decode-step kernels (``ap_add_rmsnorm``, ``ap_silu_mul``,
-``ap_decode_attention``): argument checks, output allocation, the current stream.
+``ap_decode_attention``, ``ap_decode_advance``): argument checks, output allocation, the current stream.
 
 The reference has no counterpart: between its linears it runs the Hugging Face modules
 (any_precision/modules/AnyPrecisionForCausalLM.py:88-97).
@@ -78,3 +78,18 @@ def decode_attention(qkv, cos_table, sin_table, kcache, vcache, pos, n_heads, sc
                                                   vcache.data_ptr(), pos.data_ptr(), out.data_ptr(), n_heads, n_kv, hd, max_len,
                                                   float(scale), _stream(qkv)), "ap_decode_attention")
     return out
+
+
+def advance(logits, pos, tok, emitted):
+    """The end of a greedy decode step on device scalars: ``t = argmax(logits)`` (first index of the maximum);
+    ``pos += 1``; ``emitted[pos] = t`` (if that row exists); ``tok = t``.  ``pos`` and ``tok`` int64 tensors of
+    one element, ``emitted`` an int64 vector."""
+    _f16(logits, "logits")
+    for t, name in ((pos, "pos"), (tok, "tok"), (emitted, "emitted")):
+        if t.dtype != torch.int64 or not t.is_cuda or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous int64 GPU tensor")
+    if pos.numel() != 1 or tok.numel() != 1 or emitted.dim() != 1:
+        raise ValueError("pos and tok hold one element each, emitted is a vector")
+    with torch.cuda.device(logits.device):
+        _capi.check(_capi.lib.ap_decode_advance(logits.data_ptr(), logits.numel(), pos.data_ptr(), tok.data_ptr(),
+                                                emitted.data_ptr(), emitted.numel(), _stream(logits)), "ap_decode_advance")

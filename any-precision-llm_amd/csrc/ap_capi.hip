@@ -290,6 +290,17 @@ int ap_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *out, long lo
     return launch_status();
 }
 
+int ap_decode_advance(const uint16_t *logits, int n, long long *pos, long long *tok, long long *emitted, int max_len,
+                      void *stream) {
+    if (!logits || !pos || !tok || !emitted) return AP_ENULL;
+    if (n < 1 || max_len < 1) return AP_ESHAPE;
+    if (!aligned16(logits)) return AP_EALIGN;
+    drain_stale_error();
+    decode_advance_kernel<<<dim3(1), dim3(kAdvanceThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        reinterpret_cast<const half_t *>(logits), n, pos, tok, emitted, max_len);
+    return launch_status();
+}
+
 int ap_decode_attention(const uint16_t *qkv, const float *cos_table, const float *sin_table, uint16_t *kcache,
                         uint16_t *vcache, const long long *pos, uint16_t *out, int n_heads, int n_kv_heads, int head_dim,
                         int max_len, float scale, void *stream) {

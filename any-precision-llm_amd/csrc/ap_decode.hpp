@@ -103,6 +103,74 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const half_t *__restrict_
     }
 }
 
+// Greedy token selection and the bookkeeping of a decode step in one workgroup:
+//     t = argmax(logits[0 .. n))  (the first index of the maximum; a NaN counts as the maximum, as torch.argmax has it);
+//     p = *pos + 1; if p < max_len: emitted[p] = t, *pos = p;  *tok = t.
+// Replaces an argmax reduction, an increment, an indexed store and a copy -- four launch-bound library kernels.
+constexpr int kAdvanceThreads = 1024;
+__global__ __launch_bounds__(kAdvanceThreads) void decode_advance_kernel(const half_t *__restrict__ logits, int n,
+                                                                        long long *pos, long long *tok, long long *emitted,
+                                                                        int max_len) {
+    __shared__ float best_v[kAdvanceThreads / kWave];
+    __shared__ int best_i[kAdvanceThreads / kWave];
+    const int tid = threadIdx.x;
+    // a > b in the order "NaN above everything, then by value, then the lower index"
+    auto better = [](float av, int ai, float bv, int bi) {
+        const bool an = av != av, bn = bv != bv;
+        if (an != bn) return an;
+        if (!an && av != bv) return av > bv;
+        return ai < bi;
+    };
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    const int nv = n / 8;  // whole 16-byte groups; the rest one by one
+    for (int g = tid; g < nv; g += kAdvanceThreads) {
+        const half8_t v = reinterpret_cast<const half8_t *>(logits)[g];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float f = (float)v[e];
+            if (better(f, g * 8 + e, bv, bi)) {
+                bv = f;
+                bi = g * 8 + e;
+            }
+        }
+    }
+    for (int i = nv * 8 + tid; i < n; i += kAdvanceThreads) {
+        const float f = (float)logits[i];
+        if (better(f, i, bv, bi)) {
+            bv = f;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        if (better(ov, oi, bv, bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((tid & (kWave - 1)) == 0) {
+        best_v[tid / kWave] = bv;
+        best_i[tid / kWave] = bi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < kAdvanceThreads / kWave; w++)
+            if (better(best_v[w], best_i[w], bv, bi)) {
+                bv = best_v[w];
+                bi = best_i[w];
+            }
+        const long long p = *pos + 1;
+        if (p >= 0 && p < max_len) {
+            emitted[p] = bi;
+            *pos = p;
+        }
+        *tok = bi;
+    }
+}
+
 // Attention of one new token at cache row pos = *pos_p, one workgroup per query head.
 //   qkv     [n_heads + 2 n_kv_heads, HD]: the token's query, key and value heads before the rotary embedding
 //   cosT, sinT [max_len, HD / 2] fp32: cos / sin of position * inverse frequency i

@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 5
+#define AP_ABI_VERSION 6
 
 enum {
     AP_OK = 0,
@@ -158,10 +158,15 @@ int ap_probe_empty(uint32_t *sink, void *stream);
  *     out   [n_heads * head_dim] = softmax(scale * q k^T) v per head, query head h reading key/value head
  *           h / (n_heads / n_kv_heads); rotary convention x * cos + rotate_half(x) * sin.
  *   head_dim 32, 64, 128 or 256; max_len <= 8192 (AP_ELIMIT beyond); a *pos outside 0 .. max_len-1 leaves every
- *   buffer untouched.  Calls that overlap on one cache race. */
+ *   buffer untouched.  Calls that overlap on one cache race.
+ * ap_decode_advance: the end of a greedy decode step, all on device scalars: t = argmax(logits[0 .. n)) (first index of
+ *   the maximum; NaN counts as the maximum, like torch.argmax); p = *pos + 1; if p < max_len: emitted[p] = t and
+ *   *pos = p; *tok = t.  One workgroup; logits 16-byte aligned. */
 int ap_add_rmsnorm(const uint16_t *h, const uint16_t *delta, const uint16_t *weight, uint16_t *h_out, uint16_t *x_out,
                    int rows, int H, float eps, void *stream);
 int ap_silu_mul(const uint16_t *gate, const uint16_t *up, uint16_t *out, long long n, void *stream);
+int ap_decode_advance(const uint16_t *logits, int n, long long *pos, long long *tok, long long *emitted, int max_len,
+                      void *stream);
 int ap_decode_attention(const uint16_t *qkv, const float *cos_table, const float *sin_table, uint16_t *kcache,
                         uint16_t *vcache, const long long *pos, uint16_t *out, int n_heads, int n_kv_heads, int head_dim,
                         int max_len, float scale, void *stream);

@@ -79,6 +79,9 @@ def test_decode_step_argument_errors_need_no_gpu():
     assert sw(K=40) == _capi.AP_ESHAPE
     assert sw(K=32 * 64 * 17) == _capi.AP_ELIMIT          # more than 16 waves per row
     assert sw(lg=fake + 4) == _capi.AP_EALIGN
+    assert L.ap_decode_advance(fake, 100, fake, None, fake, 64, None) == _capi.AP_ENULL
+    assert L.ap_decode_advance(fake, 0, fake, fake, fake, 64, None) == _capi.AP_ESHAPE
+    assert L.ap_decode_advance(fake + 2, 100, fake, fake, fake, 64, None) == _capi.AP_EALIGN
     assert L.ap_silu_mul(fake, None, fake, 64, None) == _capi.AP_ENULL
     assert L.ap_silu_mul(fake, fake, fake, 12, None) == _capi.AP_ESHAPE
     assert L.ap_silu_mul(fake, fake, fake + 4, 64, None) == _capi.AP_EALIGN

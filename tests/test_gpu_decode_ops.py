@@ -178,3 +178,32 @@ def test_fused_step_at_llama3_8b_width_with_grouped_kv_heads():
             if (top2[0] - top2[1]).item() <= 2 * tol:
                 fused.tok.copy_(stock.tok)
                 fused.emitted.copy_(stock.emitted)
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 320, 32000, 128256 + 3])
+def test_advance_is_argmax_and_bookkeeping(n):
+    """ap_decode_advance against torch.argmax (first index of the maximum, NaN as the maximum) and the three
+    scalar updates it replaces; a position at the end of the buffer moves nothing but the token."""
+    from any_precision_amd.decode_ops import advance
+    g = torch.Generator(device="cuda").manual_seed(n)
+    for case in ("random", "ties", "nan", "neg_inf"):
+        logits = torch.randn((1, n), device="cuda", generator=g).half()
+        if case == "ties":
+            logits = (logits * 2).round() / 2                      # many equal maxima
+        elif case == "nan" and n > 2:
+            logits[0, n // 2] = float("nan")
+            logits[0, n - 1] = float("nan")
+        elif case == "neg_inf":
+            logits.fill_(float("-inf"))
+        print(f"advance n={n} {case}", flush=True)
+        want = int(torch.argmax(logits, dim=-1).item())
+        pos = torch.tensor([5], device="cuda")
+        tok = torch.tensor([-1], device="cuda")
+        emitted = torch.full((16,), -7, device="cuda")
+        advance(logits, pos, tok, emitted)
+        assert int(tok.item()) == want and int(pos.item()) == 6 and int(emitted[6].item()) == want
+        assert (emitted[:6] == -7).all() and (emitted[7:] == -7).all()
+        pos.fill_(15)                                              # no row 16: only the token changes
+        tok.fill_(-1)
+        advance(logits, pos, tok, emitted)
+        assert int(tok.item()) == want and int(pos.item()) == 15 and int(emitted[15].item()) == -7
