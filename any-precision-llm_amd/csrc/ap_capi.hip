@@ -624,10 +624,11 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     // it that shape) wherever long_rows_want_four says so, except that at M = 3 on rows of 7 waves or more the
     // row-streaming kernel is 3-15 % faster still at up to 4 bits, and at M = 4 the 4x4x4 kernel keeps 3 bits
     // (4096 x 14336, 8192 x 28672: 9 % faster than four rows).
-    const bool four = knob(kGemvRows) <= 0 && knob(kMatmulMfma4) <= 1 && geo->wpl == 1 && long_rows_want_four(M, K);
+    const bool four = knob(kGemvRows) <= 0 && knob(kMatmulMfma4) <= 1 && M < knob(kMatmulMfmaFrom) && geo->wpl == 1 &&
+                      long_rows_want_four(M, K);
     // narrow linears (k/v projections with grouped heads) at 2..4 rows: the fine-grained kernel, 5-15 % on 1024 x 8192,
     // 5-9 % on 1024 x 4096 at 3-4 rows and up to 4 bits
-    if (count == 1 && fine_mode == 1 && fits_f && N[0] <= 2048 &&
+    if (count == 1 && fine_mode == 1 && fits_f && N[0] <= 2048 && M < knob(kMatmulMfmaFrom) &&
         ((K >= 8192 && M >= 2 && M <= 4) || (M >= 3 && M <= 4 && w_bits <= 4)))
         return all(AP_ROUTE_FINE);
     if (four) {

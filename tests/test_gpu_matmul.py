@@ -188,9 +188,10 @@ def test_group_argument_errors(ext):
 
 
 def test_every_kernel_for_small_batches_agrees_with_the_oracle(ext, oracle):
-    """ap_matmul_kbit picks between the dot-product kernel and the 4x4x4 matrix-core kernel by shape and
-    bit-width; the tuning knob matmul_mfma4 forces either (0 never, 2 wherever it fits), so each is run
-    on shapes the default rule would give to the other."""
+    """ap_matmul_kbit picks between the dot-product kernel, the 4x4x4 and the 16x16x32 matrix-core kernels by shape,
+    rows and bit-width; the tuning knobs force each (matmul_mfma4: 0 never, 2 wherever it fits; matmul_mfma_from:
+    the row count from which the 16x16x32 kernel runs, 9 = never), so each is run on shapes the default rule
+    would give to another."""
     from any_precision_amd import _capi
     for N, K in ((40, 2080), (2056, 1024), (9, 11008)):
         L = make(N, K, seed=N)
@@ -204,6 +205,12 @@ def test_every_kernel_for_small_batches_agrees_with_the_oracle(ext, oracle):
                     with _capi.tuning(matmul_mfma4=mode):
                         got = ext.matmul_kbit(xg, q, luts[b], b)
                     assert_close_gemv(got, want, f"mfma4={mode} N={N} K={K} b={b} M={M}")
+                for start, route in ((2, "mfma16"), (9, "dot")):
+                    print(f"forced kernel mfma_from={start} N={N} K={K} b={b} M={M}", flush=True)
+                    with _capi.tuning(matmul_mfma4=0, matmul_mfma_from=start, gemv_stream=0, gemv_fine=0):
+                        assert _capi.matmul_route(M, N, K, b) == route
+                        got = ext.matmul_kbit(xg, q, luts[b], b)
+                    assert_close_gemv(got, want, f"mfma_from={start} N={N} K={K} b={b} M={M}")
 
 
 # (rows, elements per row): tails (K % 1024 != 0), one word group, one/several waves per row, many rows
