@@ -124,14 +124,26 @@ __global__ __launch_bounds__(kAdvanceThreads) void decode_advance_kernel(const h
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     const int nv = n / 8;  // whole 16-byte groups; the rest one by one
-    for (int g = tid; g < nv; g += kAdvanceThreads) {
-        const half8_t v = reinterpret_cast<const half8_t *>(logits)[g];
+    constexpr int AHEAD = 4;  // 16-byte groups requested together: the scan is one chain of load latencies otherwise
+    for (int g0 = tid; g0 < nv; g0 += AHEAD * kAdvanceThreads) {
+        half8_t v[AHEAD];
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float f = (float)v[e];
-            if (better(f, g * 8 + e, bv, bi)) {
-                bv = f;
-                bi = g * 8 + e;
+        for (int a = 0; a < AHEAD; a++) {
+            const int g = g0 + a * kAdvanceThreads;
+            v[a] = reinterpret_cast<const half8_t *>(logits)[g < nv ? g : g0];
+        }
+#pragma unroll
+        for (int a = 0; a < AHEAD; a++) {
+            const int g = g0 + a * kAdvanceThreads;
+            if (g < nv) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float f = (float)v[a][e];
+                    if (better(f, g * 8 + e, bv, bi)) {
+                        bv = f;
+                        bi = g * 8 + e;
+                    }
+                }
             }
         }
     }
