@@ -947,8 +947,8 @@ def decode_tokens(args, torch, _capi, synth):
         "data": "synthetic (random-init weights, random prompt ids)",
         "config": {"workload": f"greedy decode of {new_tokens} tokens after a {prompt_len}-token prompt, batch 1, "
                                "32 layers / hidden 4096 / FFN 11008 / 32 heads / vocab 32000; decode step replayed "
-                               "from one HIP graph, 8 launches per layer, all this library's (7 linears in 4 launches, "
-                               "add + RMSNorm twice, rotary + cache append + attention, SiLU * up); argmax and the position / token "
+                               "from one HIP graph, 7 launches per layer, all this library's (7 linears in 4 launches, "
+                               "add + RMSNorm twice, rotary + cache append + attention; SiLU * up rides on the gate/up launch); argmax and the position / token "
                                "bookkeeping are one library kernel; embedding lookup and head are PyTorch ops"},
         "per_w_bits": rows}))
 
