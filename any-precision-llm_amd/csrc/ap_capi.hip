@@ -118,7 +118,7 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     if (S > kGemvMaxSeg) return AP_ELIMIT;
     // One row per workgroup until that would launch more than target_waves waves, then two
     // (the second row reuses the activation registers; more rows lengthen the compute
-    // tail).  From M = 3 on the activations are the larger load: always two rows.
+    // tail).  From M = 3 on the activations are the larger load: at least two rows (four in the cases below).
     // At 3-4 bits (least work per wave) and for a single linear at two activation rows the switch comes at three quarters of that:
     // 5120 x 5120 (15360 waves) is 8-15 % faster with two rows there (M = 1: within 3 % either way from 5 bits
     // on); 4096 x 4096 (8192 waves) keeps one.

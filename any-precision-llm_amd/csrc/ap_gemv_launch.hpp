@@ -24,7 +24,7 @@ struct GemvMembers {
 struct GemvGeometry {
     int wpl;   // words per lane per plane (1 or 2)
     int S;     // K-segments = waves per workgroup
-    int R;     // rows per workgroup (1, 2, or 4 at one activation row)
+    int R;     // rows per workgroup (1 up to two activation rows, 2, or 4 up to four activation rows)
     int grid;  // workgroups (of all members together)
 };
 
