@@ -47,6 +47,8 @@ lib.ap_probe_empty.argtypes = [_vp, _vp]
 lib.ap_probe_empty.restype = _ci
 lib.ap_matmul_kbit_route.argtypes = [_ci, _ci, _ci, _ci, _pi]
 lib.ap_matmul_kbit_route.restype = _ci
+lib.ap_matmul_kbit_group_route.argtypes = [_ci, _pi, _ci, _ci, _ci, _pi, _pi]
+lib.ap_matmul_kbit_group_route.restype = _ci
 lib.ap_matmul_kbit_swiglu.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 lib.ap_matmul_kbit_swiglu.restype = _ci
 lib.ap_add_rmsnorm.argtypes = [_vp, _vp, _vp, _vp, _vp, _ci, _ci, ctypes.c_float, _vp]
@@ -68,7 +70,7 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
     )
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
-           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_probe_write", "ap_matmul_kbit_route",
+           "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_probe_write", "ap_matmul_kbit_route", "ap_matmul_kbit_group_route",
            "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu", "ap_decode_advance")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
@@ -109,6 +111,16 @@ def matmul_route(M: int, N: int, K: int, w_bits: int) -> str:
     r = ctypes.c_int()
     check(lib.ap_matmul_kbit_route(M, N, K, w_bits, ctypes.byref(r)), "ap_matmul_kbit_route")
     return ROUTES[r.value]
+
+
+def matmul_group_route(M: int, rows, K: int, w_bits: int):
+    """(kernel name per member, weight rows per workgroup of the joint dot-product launch) for a set of linears."""
+    n = len(rows)
+    r = (ctypes.c_int * n)()
+    per_wg = ctypes.c_int()
+    check(lib.ap_matmul_kbit_group_route(n, (ctypes.c_int * n)(*rows), M, K, w_bits, r, ctypes.byref(per_wg)),
+          "ap_matmul_kbit_group_route")
+    return [ROUTES[v] for v in r], per_wg.value
 
 
 def set_tuning(name: str, value: int) -> None:

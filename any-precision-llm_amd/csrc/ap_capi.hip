@@ -585,9 +585,131 @@ int run_gemv4(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, u
     return launch_status();
 }
 
-// Which kernel serves each of `count` linears that share x, M, K and w_bits (route[g] = AP_ROUTE_*), and the
-// geometry of the grouped dot-product launch when that is the answer (then every member has AP_ROUTE_DOT).
-// `out` may be null (route queries): the output pointers are then taken to be aligned.
+// ---------------------------------------------------------------------------------------------------------------
+// Routing: which kernel serves each of `count` linears that share x, M, K and w_bits.
+//
+// Every rule below is a threshold fitted to measurements on the linears of the Llama-2-7B / Llama-3-8B / 13B / 70B
+// decoder layers (and their q/k/v and gate/up sets), cold weights, two runs each; `bench.py --workload
+// routing_audit` re-measures the default choice against every alternative.  Three parts:
+//   forced_route     a kernel forced by a tuning knob (tests, sweeps);
+//   few_rows_route   M below the knob matmul_mfma_from (1..4 by default): the dot-product family and the 4x4x4 kernel;
+//   many_rows_route  M from that knob on (5..8): the matrix-core kernels, and the dot-product kernel where it still wins.
+// The dot-product kernels other than gemv_kbit_kernel serve one linear per launch and stay within +-6 % of it on every
+// shape -- a launch is bound by its latency chain (dispatch, first loads, table staging, last compute, segment sums)
+// and by what the memory system delivers to a burst of requests, not by the instruction count -- so they are used
+// only where they won by 3 % or more.
+
+struct RouteQuery {
+    int M, count, K, w_bits;
+    const int *N;
+    int lo, hi;        // fewest / most rows of a member
+    long long rows;    // all members together
+    bool fits_persist, fits_fine, fits_stream;  // every member can run that kernel
+    const GemvGeometry *geo;                    // of the joint dot-product launch
+};
+
+bool single(const RouteQuery &q) { return q.count == 1; }
+
+// The 4x4x4 kernel's own limits (word groups per wave, waves per workgroup).
+bool mfma4_fits(const RouteQuery &q) {
+    const int W = q.K >> 5;
+    if (q.M < 2 || q.M > 8) return false;
+    return q.M <= 4 ? W <= 16 * 4 * kGemv4MaxSeg : W <= 16 * kGemv4MaxSegTwo;
+}
+
+// Knobs at 2 force their kernel wherever it fits.  Returns a route or -1.
+int forced_route(const RouteQuery &q) {
+    if (knob(kGemvPersist) >= 2 && q.fits_persist) return AP_ROUTE_PERSIST;  // never a default: slower on every shape
+    if (knob(kGemvFine) >= 2 && q.fits_fine) return AP_ROUTE_FINE;
+    if (knob(kGemvStream) >= 2 && q.fits_stream) return AP_ROUTE_STREAM;
+    return -1;
+}
+
+// M = 1..4.  One route for the whole set.
+int few_rows_route(const RouteQuery &q) {
+    const int M = q.M, K = q.K, b = q.w_bits;
+    const bool fine_ok = knob(kGemvFine) == 1 && q.fits_fine, stream_ok = knob(kGemvStream) == 1 && q.fits_stream;
+    const int m4 = knob(kMatmulMfma4);
+    // narrow linears (k/v projections with grouped heads) at 2..4 rows: the fine-grained kernel, 5-15 % on 1024 x 8192,
+    // 5-9 % on 1024 x 4096 at 3-4 rows and up to 4 bits
+    if (single(q) && fine_ok && q.lo <= 2048 && ((K >= 8192 && M >= 2) || (M >= 3 && b <= 4))) return AP_ROUTE_FINE;
+    // long rows at 2..4 rows: gemv_kbit_kernel with four rows per workgroup (gemv_geometry shapes it so) wherever
+    // long_rows_want_four says -- except M = 3 on rows of 7 waves or more at up to 4 bits (row-streaming kernel,
+    // another 3-15 %) and M = 4 at 3 bits (4x4x4 kernel, 9 % on 4096 x 14336 and 8192 x 28672)
+    if (knob(kGemvRows) <= 0 && m4 <= 1 && q.geo->wpl == 1 && long_rows_want_four(M, K)) {
+        if (single(q) && M == 3 && b <= 4 && q.geo->S >= 7 && stream_ok) return AP_ROUTE_STREAM;
+        if (!(M == 4 && b == 3 && m4 == 1)) return AP_ROUTE_DOT;
+    }
+    if (single(q)) {
+        const bool wide = q.lo >= 8192 && K <= 4096;  // gate/up of the 7B / 8B models
+        // row-streaming kernel (fewest waves and instructions): 3 bits at one row on wide linears (3-5 %), 3-4 bits at
+        // two rows on rows of >= 8192 elements that long_rows_want_four left alone (10-14 %)
+        if (stream_ok && ((M == 1 && wide && b == 3) || (M == 2 && K >= 8192 && b <= 4))) return AP_ROUTE_STREAM;
+        // fine-grained row-pair kernel (half the waves): 6-7 bits at one row on wide linears (3-6 %; at 8 bits one row per
+        // workgroup of gemv_kbit_kernel is faster still), 6-8 bits at four rows on rows of >= 8192 elements (6-15 %; at
+        // 6 bits on rows of up to 12288 elements the 4x4x4 kernel is 13 % faster and takes over)
+        if (fine_ok && ((M == 1 && wide && (b == 6 || b == 7)) || (M == 4 && K >= 8192 && b >= (K <= 12288 ? 7 : 6))))
+            return AP_ROUTE_FINE;
+    }
+    // The 4x4x4 matrix-core kernel (cost per weight flat in M, one linear per launch): 3 and 4 rows on single linears with
+    // enough rows to fill the chip, at up to 5 bits, and for 4 rows at every bit-width while a row fits one word
+    // group per lane (K <= 8192; 6 bits up to 12288): 10-40 % faster than the dot-product kernel.  Not for sets (one
+    // dot-product launch with four rows per workgroup beats a launch per member by 15-45 %) and not where
+    // mid_rows_want_four says.
+    if (m4 >= 1 && M >= 2 && mfma4_fits(q)) {
+        if (m4 >= 2) return AP_ROUTE_MFMA4;
+        const bool bits_ok = (M == 3 && b <= 5) || (M == 4 && (b <= 5 || K <= 8192 || (b == 6 && K <= 12288)));
+        if (single(q) && !mid_rows_want_four(M, K, b) && bits_ok && q.rows >= 2048) return AP_ROUTE_MFMA4;
+    }
+    return AP_ROUTE_DOT;
+}
+
+// M = 5..8 under default knobs: where the dot-product kernel (cost linear in M, one launch for all members) still
+// beats the matrix-core kernels (cost flat in M, one launch per member, 16 rows per workgroup):
+//  - a linear of at most 2048 rows (k/v projections with grouped heads: 64-128 workgroups of the MFMA kernel): 10-54 %
+//    faster at every M and bit-width; a set with such a member 6-50 % (at M >= 7 on rows of more than 4096 elements
+//    only from 5 bits on);
+//  - 7-8 bits on linears of >= 5120 rows of more than 4096 elements, where the MFMA kernel is at its worst (5120 x
+//    5120, 13824 x 5120, 8192 x 8192, 28672 x 8192): 7-41 % at M = 5..7 at 8 bits (M = 8 too on rows of 5120
+//    elements; M = 5 only on rows of 8193..16384: 5120 x 13824, 22 %; never beyond) and 9-20 % at M = 5 at 7 bits;
+//    5120 x 5120 at M = 5 from 5 bits on (14-16 %);
+//  - sets: at 8 bits on rows of 4097..8192 elements at every M (3-32 %); at M = 5 at 8 bits (8-46 %) and from 5 bits
+//    on when no member has more than 8192 rows (15-37 %).
+bool dot_beats_mfma(const RouteQuery &q) {
+    const int M = q.M, K = q.K, b = q.w_bits;
+    if (q.geo->wpl != 1) return false;
+    if (single(q)) {
+        if (q.lo <= 2048) return true;
+        if (K <= 4096 || q.lo < 5120) return false;
+        if (b == 8) return K <= 8192 ? (M <= 7 || K <= 5120) : (M == 5 && K <= 16384);
+        if (b == 7) return M == 5 && K <= 8192;
+        return M == 5 && b >= 5 && (long long)q.lo * K <= 32LL << 20;
+    }
+    if (q.lo <= 2048 && (M <= 6 || K <= 4096 || b >= 5)) return true;
+    if (b == 8 && K > 4096 && K <= 8192) return true;
+    return M == 5 && (b == 8 || (b >= 5 && q.hi <= 8192));
+}
+
+// M from the knob matmul_mfma_from on.  Routes per member (the matrix-core kernels serve one linear per launch).
+void many_rows_route(const RouteQuery &q, int *route) {
+    const int m4 = knob(kMatmulMfma4);
+    const bool defaults = knob(kMatmulMfmaFrom) == 5 && m4 <= 1;
+    if (defaults && q.M >= 5 && dot_beats_mfma(q)) {
+        for (int g = 0; g < q.count; g++) route[g] = AP_ROUTE_DOT;
+        return;
+    }
+    // 4x4x4 kernel with two groups of four activation rows (5..8 rows): on wide linears (16 rows per workgroup) with
+    // rows of 3072..4096 elements (5..8 waves per workgroup) from 4 bits on it is 5-20 % faster than the 16x16x32
+    // kernel; shorter and longer rows and narrower linears measured slower, and at 3 bits the 16x16x32 kernel with its
+    // pair-table lookups is 4-18 % faster (11008 / 14336 x 4096).
+    for (int g = 0; g < q.count; g++) {
+        const bool pays = q.M >= 5 && q.K >= 3072 && q.N[g] >= 10240 && q.w_bits >= 4;
+        route[g] = m4 >= 1 && mfma4_fits(q) && (m4 >= 2 || pays) ? AP_ROUTE_MFMA4 : AP_ROUTE_MFMA16;
+    }
+}
+
+// route[g] = AP_ROUTE_* per member, and in *geo / *mem the geometry of the joint dot-product launch (used when every
+// member has AP_ROUTE_DOT).  `out` may be null (route queries): the output pointers are then taken to be aligned.
 int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *const *out, GemvGeometry *geo,
                 GemvMembers *mem, int *route) {
     const int rc = gemv_geometry(M, N, count, K, w_bits, geo, mem);
@@ -599,119 +721,21 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     // a row longer than one workgroup of the dot-product kernel covers (65536 elements at M <= 2, 32768
     // beyond): the MFMA kernel walks rows of any length
     if (rc == AP_ELIMIT) return all(AP_ROUTE_MFMA16);
-    // Three more dot-product kernels (one linear per launch each), all with the same lookups and sums as
-    // gemv_kbit_kernel but a different split of the work over waves.  Measured on cold planes they stay
-    // within +-6 % of it on every 7B/8B/70B shape -- a launch is bound by its latency chain (dispatch,
-    // first loads, table staging, last compute, segment sums) and by what the memory system delivers to a
-    // burst of requests, not by the instruction count -- so mode 1 uses them only where they won by 3 % or
-    // more on two boxes, for single linears:
-    //  - row-streaming kernel (fewest waves and instructions): 3 bits at batch 1 on linears of >= 8192
-    //    rows of <= 4096 elements (gate/up of the 7B/8B models: 3-5 %), 3-4 bits at batch 2 on rows of
-    //    >= 8192 elements (10-14 %);
-    //  - fine-grained row-pair kernel (half the waves of gemv_kbit_kernel): 6-7 bits at batch 1 on the
-    //    same wide linears (3-6 %; at 8 bits gemv_kbit_kernel with one row per workgroup is faster still),
-    //    6-8 bits at batch 4 on rows of >= 8192 elements (6-15 %; at 6 bits on rows of up to 12288 elements the
-    //    4x4x4 kernel is 13 % faster and takes over).
-    // Mode 2 of a knob forces its kernel wherever it fits (tests, sweeps); mode 0 switches it off.
-    const int persist_mode = knob(kGemvPersist), fine_mode = knob(kGemvFine), stream_mode = knob(kGemvStream);
-    bool fits_r = true, fits_f = true, fits_p = true;
+    RouteQuery q = {M, count, K, w_bits, N, N[0], N[0], 0, true, true, true, geo};
     for (int g = 0; g < count; g++) {
         const uint16_t *o = out ? out[g] : nullptr;
-        fits_r = fits_r && gemvr_fits(M, N[g], K);
-        fits_f = fits_f && gemvf_fits(o, M, N[g], K);
-        fits_p = fits_p && gemvp_fits(o, M, N[g], K);
+        q.lo = N[g] < q.lo ? N[g] : q.lo;
+        q.hi = N[g] > q.hi ? N[g] : q.hi;
+        q.rows += N[g];
+        q.fits_persist = q.fits_persist && gemvr_fits(M, N[g], K);
+        q.fits_fine = q.fits_fine && gemvf_fits(o, M, N[g], K);
+        q.fits_stream = q.fits_stream && gemvp_fits(o, M, N[g], K);
     }
-    if (persist_mode >= 2 && fits_r) return all(AP_ROUTE_PERSIST);  // never the default: slower on every shape
-    if (fine_mode >= 2 && fits_f) return all(AP_ROUTE_FINE);
-    if (stream_mode >= 2 && fits_p) return all(AP_ROUTE_STREAM);
-    // Long rows at 2..4 activation rows: the dot-product kernel with four rows per workgroup (gemv_geometry gives
-    // it that shape) wherever long_rows_want_four says so, except that at M = 3 on rows of 7 waves or more the
-    // row-streaming kernel is 3-15 % faster still at up to 4 bits, and at M = 4 the 4x4x4 kernel keeps 3 bits
-    // (4096 x 14336, 8192 x 28672: 9 % faster than four rows).
-    const bool four = knob(kGemvRows) <= 0 && knob(kMatmulMfma4) <= 1 && M < knob(kMatmulMfmaFrom) && geo->wpl == 1 &&
-                      long_rows_want_four(M, K);
-    // narrow linears (k/v projections with grouped heads) at 2..4 rows: the fine-grained kernel, 5-15 % on 1024 x 8192,
-    // 5-9 % on 1024 x 4096 at 3-4 rows and up to 4 bits
-    if (count == 1 && fine_mode == 1 && fits_f && N[0] <= 2048 && M < knob(kMatmulMfmaFrom) &&
-        ((K >= 8192 && M >= 2 && M <= 4) || (M >= 3 && M <= 4 && w_bits <= 4)))
-        return all(AP_ROUTE_FINE);
-    if (four) {
-        if (count == 1 && M == 3 && w_bits <= 4 && geo->S >= 7 && stream_mode == 1 && fits_p) return all(AP_ROUTE_STREAM);
-        if (!(M == 4 && w_bits == 3 && knob(kMatmulMfma4) == 1)) return all(AP_ROUTE_DOT);
-    }
-    if (count == 1) {
-        const bool wide = N[0] >= 8192 && K <= 4096;
-        if (stream_mode == 1 && fits_p && ((M == 1 && wide && w_bits == 3) || (M == 2 && K >= 8192 && w_bits <= 4)))
-            return all(AP_ROUTE_STREAM);
-        if (fine_mode == 1 && fits_f && ((M == 1 && wide && (w_bits == 6 || w_bits == 7)) || (M == 4 && K >= 8192 && w_bits >= (K <= 12288 ? 7 : 6))))
-            return all(AP_ROUTE_FINE);
-    }
-    // The 4x4x4 matrix-core kernel, whose cost per weight does not grow with M, where it measured
-    // faster than both other kernels (it serves one linear per launch):
-    //  - 3 and 4 activation rows on linears with enough rows to fill the chip (8 per workgroup), at up
-    //    to 5 bits, and for 4 rows at every bit-width while a row fits one word group per lane
-    //    (K <= 8192): 10-40 % faster than the dot-product kernel;
-    //  - 5..8 activation rows on wide linears (16 rows per workgroup) with rows of 3072..4096 elements
-    //    (5..8 waves per workgroup) from 4 bits on: 5-20 % faster than the 16x16x32 MFMA kernel.  Shorter and
-    //    longer rows and narrower linears measured slower, and at 3 bits the MFMA kernel with its pair-table
-    //    lookups is 4-18 % faster (11008 / 14336 x 4096).
-    const int m4 = knob(kMatmulMfma4);
-    long long rows = 0;
-    for (int g = 0; g < count; g++) rows += N[g];
-    // 5..8 activation rows where the dot-product kernel (cost linear in M, one launch for all members) still beats
-    // the matrix-core kernels (cost flat in M, one launch per member, 16 rows per workgroup).  Swept at M = 5..8,
-    // 3..8 bits, on the 7B / 8B / 13B / 70B linears and their q/k/v and gate/up sets (default knobs only):
-    //  - a linear of at most 2048 rows (k/v projections with grouped heads: 64-128 workgroups of the MFMA kernel):
-    //    10-54 % faster at every M and bit-width; a set with such a member 6-50 % (at M >= 7 on rows of more than
-    //    4096 elements only from 5 bits on);
-    //  - 7-8 bits on linears of >= 5120 rows of more than 4096 elements, where the MFMA kernel is at its worst (5120 x
-    //    5120, 13824 x 5120, 8192 x 8192, 28672 x 8192): 7-41 % at M = 5..7 at 8 bits (M = 8 too on rows of 5120
-    //    elements; M = 5 only on rows of 8193..16384: 5120 x 13824, 22 %; never beyond) and 9-20 % at M = 5 at 7 bits;
-    //  - sets at M = 5: 8-46 % at 8 bits, and 15-37 % from 5 bits on when no member has more than 8192 rows.
-    auto dot_beats_mfma = [&]() {
-        if (M < 5 || M > 8 || knob(kMatmulMfmaFrom) != 5 || m4 >= 2 || geo->wpl != 1) return false;
-        int lo = N[0], hi = N[0];
-        for (int g = 1; g < count; g++) {
-            lo = N[g] < lo ? N[g] : lo;
-            hi = N[g] > hi ? N[g] : hi;
-        }
-        if (count == 1) {
-            if (lo <= 2048) return true;
-            if (K <= 4096 || lo < 5120) return false;
-            if (w_bits == 8) return K <= 8192 ? (M <= 7 || K <= 5120) : (M == 5 && K <= 16384);
-            if (w_bits == 7) return M == 5 && K <= 8192;
-            return M == 5 && w_bits >= 5 && (long long)lo * K <= 32LL << 20;  // 5120 x 5120: 14-16 %
-        }
-        if (lo <= 2048 && (M <= 6 || K <= 4096 || w_bits >= 5)) return true;
-        if (w_bits == 8 && K > 4096 && K <= 8192) return true;  // every M: 3-32 % (13B / 70B sets)
-        return M == 5 && (w_bits == 8 || (w_bits >= 5 && hi <= 8192));
-    };
-    if (dot_beats_mfma()) return all(AP_ROUTE_DOT);
-    auto use4 = [&](int n) {
-        const int W = K >> 5;
-        if (m4 == 0 || M < 2 || M > 8) return false;
-        if (M <= 4) {  // decided for the group as a whole, by its mean row count
-            if (W > 16 * 4 * kGemv4MaxSeg) return false;  // at most 4 word groups per wave, 16 waves
-            if (m4 >= 2) return true;
-            if (count > 1) return false;  // several linears: one dot-product launch with four rows per workgroup beats a launch each
-            if (mid_rows_want_four(M, K, w_bits)) return false;
-            return ((M == 3 && w_bits <= 5) || (M == 4 && (w_bits <= 5 || K <= 8192 || (w_bits == 6 && K <= 12288)))) &&
-                   rows >= 2048LL * count;
-        }
-        if (W > 16 * kGemv4MaxSegTwo) return false;
-        if (m4 >= 2) return true;
-        return K >= 3072 && n >= 10240 && w_bits >= 4;  // per member; the others go to the MFMA kernel
-    };
-    bool any4 = false;
-    for (int g = 0; g < count; g++) any4 |= use4(N[g]);
-    if (any4) {
-        for (int g = 0; g < count; g++) route[g] = use4(N[g]) ? AP_ROUTE_MFMA4 : AP_ROUTE_MFMA16;
-        return AP_OK;
-    }
-    // From 5 activation rows on, the 16x16x32 MFMA kernel (cost flat in M up to 16 rows) is faster than
-    // the dot-product kernel (cost linear in M) on most shapes and bit-widths; one linear per launch.
-    if (M >= knob(kMatmulMfmaFrom)) return all(AP_ROUTE_MFMA16);
-    return all(AP_ROUTE_DOT);
+    const int forced = forced_route(q);
+    if (forced >= 0) return all(forced);
+    if (M < knob(kMatmulMfmaFrom)) return all(few_rows_route(q));
+    many_rows_route(q, route);
+    return AP_OK;
 }
 
 }  // namespace
@@ -829,6 +853,15 @@ int ap_matmul_kbit_route(int M, int N, int K, int w_bits, int *route) {
     if (!route) return AP_ENULL;
     GemvGeometry geo;
     return plan_matmul(M, &N, 1, K, w_bits, nullptr, &geo, nullptr, route);
+}
+
+int ap_matmul_kbit_group_route(int count, const int *N, int M, int K, int w_bits, int *route, int *rows) {
+    if (!N || !route) return AP_ENULL;
+    if (count < 1 || count > kGemvMaxGroup) return AP_ELIMIT;
+    GemvGeometry geo = {};  // rows stays 0 when no dot-product launch can serve the set
+    const int rc = plan_matmul(M, N, count, K, w_bits, nullptr, &geo, nullptr, route);
+    if (rc == AP_OK && rows) *rows = geo.R;
+    return rc;
 }
 
 }  // extern "C"

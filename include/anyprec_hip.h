@@ -117,6 +117,10 @@ enum {
     AP_ROUTE_MFMA16 = 5   /* gemm_kbit_kernel: 16x16x32 matrix-core kernel                               */
 };
 int ap_matmul_kbit_route(int M, int N, int K, int w_bits, int *route);
+/* The same for a set of `count` linears given to ap_matmul_kbit_group: route[g] per member (all AP_ROUTE_DOT = one
+ * launch for the set; anything else = a launch per member) and, if `rows` is not NULL, the weight rows per workgroup
+ * the dot-product kernel would use for the set. */
+int ap_matmul_kbit_group_route(int count, const int *N, int M, int K, int w_bits, int *route, int *rows);
 
 /* Test and measurement hook, no counterpart in the reference: overrides one launch-heuristic knob
  * (which kernel variant serves a shape, grid sizes) for the whole process, so that tests can force

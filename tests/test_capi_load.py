@@ -144,6 +144,15 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_route(8, 1024, 4096, 3) == "dot"                # too few rows for 16 per workgroup
     assert _capi.matmul_route(5, 5120, 5120, 8) == "dot" and _capi.matmul_route(8, 8192, 8192, 8) == "mfma16"
     assert _capi.matmul_route(5, 8192, 28672, 8) == "mfma16" and _capi.matmul_route(3, 1024, 8192, 5) == "fine"
+    # sets of linears (ap_matmul_kbit_group): one dot-product launch up to 4 rows, four weight rows per workgroup at 3-4
+    assert _capi.matmul_group_route(1, [4096, 4096, 4096], 4096, 3) == (["dot"] * 3, 4)
+    assert _capi.matmul_group_route(1, [4096, 4096, 4096], 4096, 8) == (["dot"] * 3, 1)
+    assert _capi.matmul_group_route(3, [4096, 1024, 1024], 4096, 5) == (["dot"] * 3, 4)
+    assert _capi.matmul_group_route(8, [4096, 1024, 1024], 4096, 3)[0] == ["dot"] * 3       # a narrow member
+    assert _capi.matmul_group_route(8, [11008, 11008], 4096, 4)[0] == ["mfma4", "mfma4"]     # a launch per member
+    assert _capi.matmul_group_route(8, [4096, 4096, 4096], 4096, 3)[0] == ["mfma16"] * 3
+    with pytest.raises(ValueError):
+        _capi.matmul_group_route(1, [64] * 5, 4096, 3)
     with _capi.tuning(matmul_mfma_from=5, matmul_mfma4=2):
         assert _capi.matmul_route(8, 1024, 4096, 3) != "dot"            # a forced kernel overrides the rule
     assert _capi.matmul_route(1, 8, 32 * 64 * 2 * 17, 4) == "mfma16"      # longer than a workgroup covers
