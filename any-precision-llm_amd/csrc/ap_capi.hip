@@ -427,7 +427,7 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     // 5 bits; and at 8 bits up to 16 activation rows gain 8-16 % wherever a wave has more than one step (rows of
     // more than 4096 elements: 5120 x 5120, 13824 x 5120, 5120 x 13824, 8192 x 8192, 8192 x 28672).
     const bool big = (long long)N * K >= 56LL << 20;
-    const bool low_bits = w_bits == 3 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (big || N < 8192));
+    const bool low_bits = w_bits <= 4 || (w_bits <= (geo.mb >= 2 ? 6 : 5) && (big || N < 8192));  // 4 bits: 11008 x 4096, 7-10 %
     const bool rb_pays = N >= 5120 && (M > 8 ? (low_bits || (w_bits == 8 && M <= 16 && K > 4096))
                                              : (M >= 5 && ((w_bits == 3 && big && N >= 8192) ||  // 14336 x 4096 at 5..8 rows: 6-18 %
                                                            (K >= 8192 && N <= 8192))));  // 5120 x 13824, 8192 x 28672, 8192 x 8192: 5-17 %
@@ -687,6 +687,7 @@ bool dot_beats_mfma(const RouteQuery &q) {
     }
     if (q.lo <= 2048 && (M <= 6 || K <= 4096 || b >= 5)) return true;
     if (b == 8 && K > 4096 && K <= 8192) return true;
+    if (M == 5 && K > 4096 && K <= 8192 && q.hi <= 8192) return true;  // q/k/v of the 13B model: 5-46 % at every bit-width
     return M == 5 && (b == 8 || (b >= 5 && q.hi <= 8192));
 }
 
@@ -732,9 +733,24 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         q.fits_stream = q.fits_stream && gemvp_fits(o, M, N[g], K);
     }
     const int forced = forced_route(q);
-    if (forced >= 0) return all(forced);
-    if (M < knob(kMatmulMfmaFrom)) return all(few_rows_route(q));
-    many_rows_route(q, route);
+    if (forced >= 0)
+        all(forced);
+    else if (M < knob(kMatmulMfmaFrom))
+        all(few_rows_route(q));
+    else
+        many_rows_route(q, route);
+    // A set is either ONE dot-product launch or, member by member, exactly what each linear would get on its own
+    // (a narrow k/v projection beside a wide q projection then still goes to the kernel that suits it).
+    bool one_launch = true;
+    for (int g = 0; g < count; g++) one_launch = one_launch && route[g] == AP_ROUTE_DOT;
+    if (count > 1 && !one_launch) {
+        for (int g = 0; g < count; g++) {
+            GemvGeometry own;
+            uint16_t *const *o = out ? out + g : nullptr;
+            const int r = plan_matmul(M, N + g, 1, K, w_bits, o, &own, nullptr, route + g);
+            if (r != AP_OK) return r;
+        }
+    }
     return AP_OK;
 }
 
@@ -824,7 +840,16 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     drain_stale_error();
-    if (route[0] == AP_ROUTE_DOT) {  // the whole set in one launch (plan_matmul gives all members this route or none)
+    bool one_launch = true;
+    for (int g = 0; g < count; g++) one_launch = one_launch && route[g] == AP_ROUTE_DOT;
+    if (count > 1 && !one_launch) {  // member by member, each as a linear of its own
+        for (int g = 0; g < count; g++) {
+            const int r = ap_matmul_kbit_group(x, 1, qweight + g, lut + g, out + g, N + g, M, K, w_bits, stream);
+            if (r != AP_OK) return r;
+        }
+        return AP_OK;
+    }
+    if (one_launch) {  // the whole set in one launch
         switch (w_bits) {
             case 3: launch_gemv<3>(M, geo, x, mem, K, st); break;
             case 4: launch_gemv<4>(M, geo, x, mem, K, st); break;

@@ -50,6 +50,8 @@ def parse_args():
                          "kernel and geometry the tuning knobs can force: where is the default not the fastest.")
     ap.add_argument("--audit-models", default="7b,8b", help="routing_audit: comma list out of 7b, 8b, 13b, 70b")
     ap.add_argument("--audit-rows", default="1,2,3,4,5,8", help="routing_audit: activation row counts")
+    ap.add_argument("--audit-sets", action="store_true", help="routing_audit: also the q/k/v and gate/up sets (ap_matmul_kbit_group)")
+    ap.add_argument("--audit-gemm", action="store_true", help="routing_audit: also ap_gemm_kbit at 16, 32, 64 rows")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -708,6 +710,12 @@ def gemv_kernel_variants(args, torch, _capi, synth):
         "value": None, "kernels": rows}))
 
 
+AUDIT_SETS = {     # linears of a decoder layer that share their input: ((rows of each member), elements per row)
+    "7b": (((4096, 4096, 4096), 4096), ((11008, 11008), 4096)),
+    "8b": (((4096, 1024, 1024), 4096), ((14336, 14336), 4096)),
+    "13b": (((5120, 5120, 5120), 5120), ((13824, 13824), 5120)),
+    "70b": (((8192, 1024, 1024), 8192), ((28672, 28672), 8192)),
+}
 AUDIT_SHAPES = {   # (rows, elements per row) of the distinct linears of a decoder layer
     "7b": ((4096, 4096), (11008, 4096), (4096, 11008)),
     "8b": ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)),
@@ -771,15 +779,93 @@ def routing_audit(args, torch, _capi, synth):
                 cases.append(case)
                 if us["default"] > 1.05 * us[best]:
                     losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
+        # the fused GEMM of ap_gemm_kbit on the same weights: one or two row blocks per workgroup, the row-walking kernel
+        for b in bits:
+            for M in ((16, 32, 64) if args.audit_gemm else ()):
+                x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+                big_out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+
+                def gemm(st):
+                    cur["j"] = (cur["j"] + 1) % P.sets
+                    rc = lib.ap_gemm_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                          big_out.data_ptr(), M, N, K, b, st)
+                    if rc != 0:
+                        raise RuntimeError(_capi.strerror(rc))
+
+                reps = min(P.sets, 16)
+                us = {"default": _graph_us(torch, side, gemm, reps)}
+                for name, knobs in (("one_block", {"gemm_walk": 0, "gemm_rb2": 0}), ("two_blocks", {"gemm_walk": 0, "gemm_rb2": 2}),
+                                    ("walking", {"gemm_walk": 2})):
+                    with _capi.tuning(**knobs):
+                        us[name] = _graph_us(torch, side, gemm, reps)
+                us["default"] = min(us["default"], _graph_us(torch, side, gemm, reps))
+                best = min((k for k in us if k != "default"), key=lambda k: us[k])
+                case = {"entry": "ap_gemm_kbit", "N": N, "K": K, "w_bits": b, "M": M, "default_us": round(us["default"], 2),
+                        "best": best, "best_us": round(us[best], 2)}
+                cases.append(case)
+                if us["default"] > 1.05 * us[best]:
+                    losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
         del P
         torch.cuda.empty_cache()
+    # sets of linears that share their input (q/k/v, gate/up) through ap_matmul_kbit_group: the default against one
+    # dot-product launch with 2 or 4 rows per workgroup and against a launch per member
+    import ctypes
+    for m in (args.audit_models.split(",") if args.audit_sets else ()):
+        for Ns, K in AUDIT_SETS[m.strip()]:
+            pools = [WeightPool(torch, N, K, max(3, int(args.pool_gb * 0.5e9 / (sum(Ns) * K)) + 1), gen, bits=bits) for N in Ns]
+            n = len(Ns)
+            arr, rows_arr = ctypes.c_void_p * n, (ctypes.c_int * n)(*Ns)
+            cur = {"j": 0}
+            for b in bits:
+                for M in Ms:
+                    x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+                    outs = arr(*[P.out.data_ptr() for P in pools])
+
+                    def group(st):
+                        cur["j"] = (cur["j"] + 1) % pools[0].sets
+                        j = cur["j"]
+                        rc = lib.ap_matmul_kbit_group(x.data_ptr(), n, arr(*[P.qweight[j].data_ptr() for P in pools]),
+                                                      arr(*[P.luts[b][j].data_ptr() for P in pools]), outs, rows_arr, M, K, b, st)
+                        if rc != 0:
+                            raise RuntimeError(_capi.strerror(rc))
+
+                    def per_member(st):
+                        cur["j"] = (cur["j"] + 1) % pools[0].sets
+                        for P in pools:
+                            rc = lib.ap_matmul_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                                    P.out.data_ptr(), M, P.N, K, b, st)
+                            if rc != 0:
+                                raise RuntimeError(_capi.strerror(rc))
+
+                    reps = min(pools[0].sets, 12)
+                    us = {"default": _graph_us(torch, side, group, reps), "launch_per_member": _graph_us(torch, side, per_member, reps)}
+                    forced = dict(dot, matmul_mfma_from=9)
+                    for name, knobs in (("one_launch_2rows", dict(forced, gemv_rows=2)), ("one_launch_4rows", dict(forced, gemv_rows=4))):
+                        if name == "one_launch_4rows" and M > 4:
+                            continue
+                        with _capi.tuning(**knobs):
+                            routes, per_wg = _capi.matmul_group_route(M, list(Ns), K, b)
+                            if set(routes) == {"dot"} and per_wg == int(name[11]):
+                                us[name] = _graph_us(torch, side, group, reps)
+                    us["default"] = min(us["default"], _graph_us(torch, side, group, reps))
+                    best = min((k for k in us if k != "default"), key=lambda k: us[k])
+                    case = {"entry": "ap_matmul_kbit_group", "N": list(Ns), "K": K, "w_bits": b, "M": M,
+                            "route": _capi.matmul_group_route(M, list(Ns), K, b)[0][0], "default_us": round(us["default"], 2),
+                            "best": best, "best_us": round(us[best], 2)}
+                    cases.append(case)
+                    if us["default"] > 1.05 * us[best]:
+                        losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
+            del pools
+            torch.cuda.empty_cache()
     within = 1 - len(losses) / len(cases)
     print(json.dumps({
         "metric": "share of (shape, rows, w_bits) cases where ap_matmul_kbit's default launch is within 5 % of the fastest forced alternative",
         "value": round(within, 4), "unit": "fraction", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None,
         "data": "synthetic", "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate",
-        "config": {"workload": f"linears of {args.audit_models} at {args.audit_rows} activation rows, w_bits 3, 4, 5, 8; cold weight "
-                               "sets; HIP graphs; alternatives forced through ap_set_tuning"},
+        "config": {"workload": f"linears of {args.audit_models} at {args.audit_rows} activation rows, w_bits 3, 4, 5, 8"
+                               + (", their q/k/v and gate/up sets" if args.audit_sets else "")
+                               + (", ap_gemm_kbit at 16, 32, 64 rows" if args.audit_gemm else "")
+                               + "; cold weight sets; HIP graphs; alternatives forced through ap_set_tuning"},
         "cases": len(cases), "worst_excess": max((l["excess"] for l in losses), default=0.0),
         "losses": sorted(losses, key=lambda l: -l["excess"]), "all_cases": cases}))
 

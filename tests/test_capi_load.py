@@ -151,6 +151,7 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_group_route(8, [4096, 1024, 1024], 4096, 3)[0] == ["dot"] * 3       # a narrow member
     assert _capi.matmul_group_route(8, [11008, 11008], 4096, 4)[0] == ["mfma4", "mfma4"]     # a launch per member
     assert _capi.matmul_group_route(8, [4096, 4096, 4096], 4096, 3)[0] == ["mfma16"] * 3
+    assert _capi.matmul_group_route(8, [8192, 1024, 1024], 8192, 3)[0] == ["mfma16", "dot", "dot"]   # each as a linear of its own
     with pytest.raises(ValueError):
         _capi.matmul_group_route(1, [64] * 5, 4096, 3)
     with _capi.tuning(matmul_mfma_from=5, matmul_mfma4=2):
