@@ -59,15 +59,17 @@ int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
 int ap_matmul_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                    uint16_t *out, int M, int N, int K, int w_bits, void *stream);
 
-/* The GEMVs of `count` (1..4) linears that share x, M, K and w_bits in ONE launch:
- * out[g][M, N[g]] = x[M,K] . dequant(qweight[g], lut[g])^T.  The arrays are host arrays of
- * `count` device pointers / row counts.  For the q/k/v and gate/up projections of a decoder
- * layer, whose launches are otherwise bound by the fixed cost of a kernel launch.  No
- * counterpart in the reference (its hook for it, fuse_layers, is a stub:
- * AnyPrecisionForCausalLM.py:168-172).  Results equal `count` calls of ap_matmul_kbit within
- * the 1e-2 bar of the path, and bit for bit whenever the same kernel serves both (always with
- * the tuning knobs gemv_stream and gemv_fine at 0: a few wide shapes otherwise go to a kernel
- * that sums in another order when called one by one).  1 <= M <= 8. */
+/* The GEMVs of `count` (1..4) linears that share x, M, K and w_bits:
+ * out[g][M, N[g]] = x[M,K] . dequant(qweight[g], lut[g])^T, in ONE launch wherever the dot-product
+ * kernel serves the set (always up to 4 activation rows; at 5..8 rows for sets with narrow members and
+ * some 5-8-bit cases, see ap_matmul_kbit_group_route), otherwise member by member exactly as
+ * ap_matmul_kbit would run each.  The arrays are host arrays of `count` device pointers / row counts.
+ * For the q/k/v and gate/up projections of a decoder layer, whose launches are otherwise bound by the
+ * fixed cost of a kernel launch.  No counterpart in the reference (its hook for it, fuse_layers, is a
+ * stub: AnyPrecisionForCausalLM.py:168-172).  Results equal `count` calls of ap_matmul_kbit within
+ * the 1e-2 bar of the path, and bit for bit whenever the same kernel serves both (always with the
+ * tuning knobs gemv_stream, gemv_fine and matmul_mfma4 at 0: some shapes otherwise go to a kernel that
+ * sums in another order when called one by one).  1 <= M <= 8. */
 int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight,
                          const uint16_t *const *lut, uint16_t *const *out, const int *N,
                          int M, int K, int w_bits, void *stream);
