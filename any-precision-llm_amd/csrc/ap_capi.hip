@@ -85,7 +85,8 @@ int check_common(int N, int K, int w_bits) {
 //   M = 3, 4: 8-40 % faster than the 4x4x4 matrix-core kernel and the two-row kernel on rows of 4 waves and of
 //          7 or more (8192, 13824, 14336, 28672 elements) at almost every bit-width -- the matrix-core kernel
 //          needs two word groups per wave there and doubles its time from 4 bits on (5120 x 13824, M = 3, 4 bits:
-//          28.9 us against 18.5) --, but 10-35 % SLOWER on rows of 11008 elements (5.4 waves), which keep their routes.
+//          28.9 us against 18.5) --, but 10-35 % SLOWER on rows of 11008 elements (workgroups of 6 waves: two of them
+//          fit a CU at the four-row kernel's register count, three at the two-row kernel's), which keep their routes.
 bool long_rows_want_four(int M, int K) {
     const int W = K >> 5, S = (W + kWave - 1) / kWave;
     if (M < 2 || M > 4 || K < 8192 || S > kGemvMaxSeg) return false;
