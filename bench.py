@@ -52,6 +52,9 @@ def parse_args():
     ap.add_argument("--audit-rows", default="1,2,3,4,5,8", help="routing_audit: activation row counts")
     ap.add_argument("--audit-sets", action="store_true", help="routing_audit: also the q/k/v and gate/up sets (ap_matmul_kbit_group)")
     ap.add_argument("--audit-gemm", action="store_true", help="routing_audit: also ap_gemm_kbit at 16, 32, 64 rows")
+    ap.add_argument("--audit-decode", action="store_true",
+                    help="llama2_7b_decode: instead of the sweep over w_bits, the decode graph re-recorded under each global "
+                         "override of the GEMV launch rules (ap_set_tuning), tokens/s against the default rules'")
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--pool", type=int, default=4, help="at least this many distinct decoder layers in the pool")
@@ -971,6 +974,42 @@ def decode_tokens(args, torch, _capi, synth):
         print(json.dumps({"metric": "batch-1 decode tokens/s, eager launches (for profiling)", "value": None, "unit": "tokens/s",
                           "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "data": "synthetic",
                           "config": {"workload": f"{prompt_len}-token prompt + 16 eager tokens, Llama-2-7B-shaped model"},
+                          "per_w_bits": rows}))
+        return
+    if args.audit_decode:
+        # the launch rules were fitted to launches timed alone; this times the whole step with one rule overridden at a time
+        overrides = [("rows_1", {"gemv_rows": 1}), ("rows_2", {"gemv_rows": 2}), ("rows_4", {"gemv_rows": 4}),
+                     ("no_stream", {"gemv_stream": 0}), ("stream_everywhere", {"gemv_stream": 2}), ("no_fine", {"gemv_fine": 0}),
+                     ("fine_everywhere", {"gemv_fine": 2}), ("no_persist", {"gemv_persist": 0}), ("persist_everywhere", {"gemv_persist": 2}),
+                     ("target_waves_8192", {"gemv_target_waves": 8192}), ("target_waves_32768", {"gemv_target_waves": 32768})]
+
+        def tokens_per_s(b, knobs):
+            dec.graphs.clear()                              # the launch geometry is fixed when the step is recorded
+            with _capi.tuning(**knobs):
+                dec.prefill(ids, b)
+                dec.capture(b)
+            dec.decode(8, b)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dec.decode(200, b)
+            torch.cuda.synchronize()
+            return 200 / (time.perf_counter() - t0)
+
+        worst = 0.0
+        for b in BITS:
+            first = tokens_per_s(b, {})
+            forced = {name: round(tokens_per_s(b, knobs), 1) for name, knobs in overrides}
+            default = max(first, tokens_per_s(b, {}))       # measured first and last
+            best = max(forced, key=forced.get)
+            worst = max(worst, forced[best] / default - 1)
+            rows.append({"w_bits": b, "default_tokens_per_s": round(default, 1), "best_override": best,
+                         "best_override_tokens_per_s": forced[best], "overrides": forced})
+        print(json.dumps({"metric": "largest gain of any single global override of the GEMV launch rules over the default rules, "
+                                    "batch-1 decode tokens/s, Llama-2-7B-shaped model", "value": round(worst, 4), "unit": "fraction",
+                          "n_gpus": 1, "higher_is_better": False, "vs_baseline": None, "data": "synthetic",
+                          "dtype": "fp16 (fp32 accumulate), u32 bitplanes",
+                          "config": {"workload": f"{prompt_len}-token prompt + 200 timed tokens per setting, decode step re-recorded "
+                                                 "into a HIP graph under each override, w_bits 3-8"},
                           "per_w_bits": rows}))
         return
     for b in BITS:
