@@ -5,7 +5,7 @@ Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]
 ``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
 ``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
 Batch dispatch: up to 8 activation rows -> ``matmul_kbit`` as in the reference (:60-64);
-9 .. 32 rows (.. 64 or 128 where ``fused_gemm_pays`` says so) -> the fused ``gemm_kbit``; beyond ->
+9 .. 32 rows (.. 64, 128 or 256 where ``fused_gemm_pays`` says so) -> the fused ``gemm_kbit``; beyond ->
 ``dequant_kbit`` + ``torch.matmul`` as in the reference.
 """
 from __future__ import annotations
@@ -24,16 +24,25 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     Llama-2-7B / Llama-3-8B / 13B / 70B layers at 3, 5, 8 bits): always up to 32 activation rows (1.3-4x at 16);
     up to 64 on linears of fewer than 8192 rows, and on larger ones at up to 5 bits -- except, on rows of more
     than 4096 elements, from 6 bits on linears of 5120 rows or more (5120 x 13824, 8 bits: 121 us against 86)
-    and from 5 bits on linears of at most 2048 rows (1024 x 8192); up to 128 on linears of fewer than 8192
-    rows of at most 4096 elements (4096 x 4096: 33-35 us against 43).  Beyond, the re-read of the
-    activations per block of weight rows costs more than materialising the weight once."""
+    and from 5 bits on linears of at most 2048 rows (1024 x 8192); up to 128 on linears of 4096..8191
+    rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).  With the tiled kernel (rows of a multiple of
+    128 elements, linears of at least 4096 rows): at 3 bits up to 256 activation rows everywhere (4096 x 4096: 26 us
+    against 39-51; 11008 x 4096: 40-57 against 57-73; 8192 x 8192: 53-79 against 82-113), at 4 bits up to 128 on rows
+    of at most 8192 elements (11008 x 4096: 52 against 57-59) and up to 256 on linears of fewer than 8192 rows of at
+    most 5120 elements (4096 x 4096: 38 against 40-51).  Beyond, one table lookup per weight and tile of activation
+    rows costs more than materialising the weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
+    if GEMM_MAX_M and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
+        if w_bits == 3:
+            return True
+        if w_bits == 4 and ((rows <= 128 and 0 < in_features <= 8192) or (out_features < 8192 and 0 < in_features <= 5120)):
+            return True
     if rows <= min(64, GEMM_MAX_M):
         if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):
             return False
         return out_features < 8192 or w_bits <= 5
-    return rows <= min(128, GEMM_MAX_M) and out_features < 8192 and 0 < in_features <= 4096
+    return rows <= min(128, GEMM_MAX_M) and 4096 <= out_features < 8192 and 0 < in_features <= 4096
 
 
 def forward_group(modules, x, precision=None, concat=False):

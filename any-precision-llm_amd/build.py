@@ -62,6 +62,7 @@ def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 8) -> str:
         units.append((os.path.join(CSRC, "ap_gemvp_inst.hip"), os.path.join(OBJDIR, f"ap_gemvp_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemm_inst.hip"), os.path.join(OBJDIR, f"ap_gemm_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemmw_inst.hip"), os.path.join(OBJDIR, f"ap_gemmw_b{b}.o"), [f"-DAP_BITS={b}"]))
+        units.append((os.path.join(CSRC, "ap_gemmt_inst.hip"), os.path.join(OBJDIR, f"ap_gemmt_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemv4_inst.hip"), os.path.join(OBJDIR, f"ap_gemv4_b{b}.o"), [f"-DAP_BITS={b}"]))
     hipcc = _hipcc()
     with ThreadPoolExecutor(max_workers=jobs) as pool:

@@ -7,6 +7,7 @@
 #include "ap_decode.hpp"
 #include "ap_dequant.hpp"
 #include "ap_gemm_launch.hpp"
+#include "ap_gemmt_launch.hpp"
 #include "ap_gemmw_launch.hpp"
 #include "ap_gemv4_launch.hpp"
 #include "ap_gemv_launch.hpp"
@@ -43,6 +44,8 @@ enum {
     kGemvPersistWaves,  // waves per CU the persistent GEMV grid aims for
     kGemmWalk,          // row-walking fused GEMM: 0 never, 1 where it pays, 2 wherever it fits
     kGemmWalkWgs,       // workgroups per CU its grid aims for
+    kGemmTiled,         // tiled fused GEMM (ap_gemm_kbit): 0 never, 1 where it pays, 2 wherever it fits
+    kGemmTile,          // > 0: blocks of 16 activation rows in its tile, 4 or 8
     kKnobCount
 };
 Knob g_knobs[kKnobCount] = {
@@ -50,7 +53,7 @@ Knob g_knobs[kKnobCount] = {
     {"matmul_mfma_from", 5},      {"gemm_split", 0},     {"matmul_mfma4", 1}, {"gemv4_groups", 0},
     {"gemm_rb2", 1},              {"gemv_stream", 1},    {"gemv_stream_waves", 24},
     {"gemv_fine", 1},             {"gemv_persist", 1},   {"gemv_persist_waves", 8},
-    {"gemm_walk", 1},             {"gemm_walk_wgs", 1},
+    {"gemm_walk", 1},             {"gemm_walk_wgs", 1},  {"gemm_tiled", 1},   {"gemm_tile", 0},
 };
 inline int knob(int k) { return __atomic_load_n(&g_knobs[k].value, __ATOMIC_RELAXED); }
 
@@ -384,6 +387,36 @@ bool gemmw_geometry(int M, int N, int K, int w_bits, GemmwGeometry *geo) {
     geo->ks = ks;
     geo->grid = (int)((nblocks + rounds - 1) / rounds);  // every workgroup walks `rounds` blocks (the last ones one fewer)
     return true;
+}
+
+// Tile of the tiled fused GEMM (ap_gemmt.hpp) for a shape; false if the kernel does not serve it.  64 weight rows x
+// 64 activation rows unless that makes several workgroups per CU: then 64 x 128, which halves the table lookups per
+// matrix instruction (measured on 4096 x 4096, 11008 / 14336 x 4096, 4096 x 11008, 5120 x 5120, 8192 x 8192 at 48..384
+// rows: the larger tile wins from about 3 workgroups of the smaller one per CU on at 3 bits, from 1.3 on at 4+ bits).
+bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
+    if ((K & 127) != 0 || (long long)M * K * 2 > 0xffffffffLL) return false;
+    const int forced = knob(kGemmTile);
+    int mbw = 4;
+    if (forced > 0) {
+        if (forced != 4 && forced != 8) return false;
+        mbw = forced;
+    } else if (M > 64) {
+        const long long small = (long long)((N + 63) / 64) * ((M + 63) / 64);
+        if (10 * small >= (w_bits == 3 ? 30LL : 13LL) * cu_count()) mbw = 8;
+    }
+    geo->mbw = mbw;
+    geo->grid_n = (N + 63) / 64;
+    geo->grid_m = (M + 16 * mbw - 1) / (16 * mbw);
+    return geo->grid_m <= 65535;
+}
+
+// Where the tiled kernel is the fastest fused form (same sweep, against the K-split kernel, which serves more than 128
+// rows in chunks of 128): always beyond 128 rows; at 3 bits from 96 rows on, from 48 on linears of at least 8192 rows of
+// at most 4096 elements (11008 x 4096 at 64 rows: 27 us against 38); at 4..8 bits from 64 rows on such linears only.
+bool gemmt_pays(int M, int N, int K, int w_bits) {
+    if (M > 128) return true;
+    const bool wide = N >= 8192 && K <= 4096;
+    return w_bits == 3 ? M >= (wide ? 48 : 96) : (wide && M >= 64);
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
@@ -805,6 +838,22 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     if (M < 1) return AP_EBATCH;
     if (!aligned16(x) || !aligned16(qweight) || !aligned16(lut)) return AP_EALIGN;
     drain_stale_error();
+    {
+        GemmtGeometry tgeo;
+        const int mode = knob(kGemmTiled);
+        if (mode > 0 && gemmt_geometry(M, N, K, w_bits, &tgeo) && (mode >= 2 || gemmt_pays(M, N, K, w_bits))) {
+            hipStream_t st = static_cast<hipStream_t>(stream);
+            switch (w_bits) {
+                case 3: launch_gemmt<3>(tgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 4: launch_gemmt<4>(tgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 5: launch_gemmt<5>(tgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 6: launch_gemmt<6>(tgeo, x, qweight, lut, out, M, N, K, st); break;
+                case 7: launch_gemmt<7>(tgeo, x, qweight, lut, out, M, N, K, st); break;
+                default: launch_gemmt<8>(tgeo, x, qweight, lut, out, M, N, K, st); break;
+            }
+            return launch_status();
+        }
+    }
     // one launch serves up to kGemmMaxM activation rows; more go in chunks of that many, in order (the planes
     // are re-read per chunk; row offsets of 128 rows keep x and out 16-byte aligned for every K and N that passed)
     for (int m0 = 0; m0 < M; m0 += kGemmMaxM) {

@@ -1,0 +1,257 @@
+// Tiled fused bitplane dequant -> MFMA GEMM for gfx950, for batches of tens to hundreds of activation rows:
+//     out[m,n] = sum_k x[m,k] * lut[n, index_b(n,k)]      (fp16 operands, fp32 accumulate)
+//
+// The reference writes the whole fp16 weight with dequant_kbit and calls torch.matmul above 8 rows
+// (any_precision/modules/AnyPrecisionLinear.py:60-62).  The K-split kernel of ap_gemm.hpp keeps the weights in
+// registers but re-reads the activations from L2 once per 16 weight rows, which bounds it from about 64 rows on.
+// Here a workgroup owns a tile of BN = 64 RB weight rows x BM = 16 MBW activation rows for the WHOLE of K:
+//   * four waves, each on its own 16 RB weight rows; a wave rebuilds its weights in registers exactly as ap_gemm.hpp
+//     does (lane = row l % 16 and word 4s + l / 16; one B operand per byte group of a word) -- no LDS round trip and
+//     one table lookup per weight and tile of activation rows;
+//   * the activations of the tile are staged ONCE per workgroup in LDS, double-buffered, 256 contiguous bytes per row
+//     and stage (byte group j of the 16 words of a step: 128 consecutive elements), and every A operand a wave reads
+//     from there feeds RB matrix instructions; the 16-byte units of a row are XOR-swizzled with the row number so
+//     that the 16 rows of an operand read hit 16 different bank groups;
+//   * accumulators (RB x MBW tiles of 16 x 16) stay in registers over the whole K loop: no K-split, no combine.
+// Per stage a wave issues 4 x RB x MBW matrix instructions between two barriers.  K must be a multiple of 128.
+#pragma once
+#include <type_traits>
+
+#include "ap_bitplane.hpp"
+#include "ap_device.hpp"
+#include "ap_gemm.hpp"
+#include "ap_gemmt_launch.hpp"
+#include "ap_lookup.hpp"
+
+namespace ap {
+
+template <int BITS, int RB, int MBW>
+__global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
+    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
+    half_t *__restrict__ out, int M, int N, int K) {
+    constexpr int NC = 1 << BITS;
+    // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 256 bytes per row).  At 4 bits that
+    // table is 1 KB per row -- too much for 64 RB rows beside the activation stages -- so 4 bits use single indices.
+    constexpr bool PAIR = BITS == 3;
+    constexpr int TB = PAIR ? LookupTable<BITS>::kBytes : 2 * NC;  // bytes of one row's table in LDS
+    constexpr int WROWS = kGemmRows * RB;                           // weight rows per wave
+    constexpr int BN = kGemmtWaves * WROWS, BM = 16 * MBW;
+    constexpr int NTHR = kGemmtWaves * kWave;
+    __shared__ __attribute__((aligned(16))) uint8_t tables[BN][TB];
+    __shared__ u32x4 xt[2][BM][16];  // [stage buffer][activation row][16-byte unit ^ (row & 15)]
+
+    const int lane = threadIdx.x;
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int tid = wv * kWave + lane;
+    const int col = lane & 15, grp = lane >> 4;
+    const int W = K >> 5;
+    const size_t plane_stride = (size_t)N * W;
+    const int nb = blockIdx.x * BN;     // first weight row of the workgroup
+    const int n0 = nb + wv * WROWS;     // ... of this wave
+    const int m0 = blockIdx.y * BM;     // first activation row of the tile
+    const int steps = (W + 15) >> 4;    // 16 words of every row per step
+    // (all workgroups walk K in the same order: those in flight then read the same columns of the activations at
+    // about the same time and share them in L2 -- walking from staggered starting steps measured 10-35 % slower)
+    auto step_at = [&](int i) { return i < steps ? i : 0; };
+
+    const uint32_t *wrow[RB];  // rows past N repeat row N-1 and are not stored
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) wrow[rb] = qweight + (size_t)min(n0 + rb * kGemmRows + col, N - 1) * W;
+    // one 16-byte load per plane: the four words 16 step + 4 grp .. + 3 (W % 4 == 0: a quad lies inside the row or
+    // past its end; then it is clamped to the last quad and never used)
+    auto fetch = [&](int step, uint32_t(&q)[RB][BITS][4]) {
+        const int w = min(16 * step + 4 * grp, W - 4);
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int p = 0; p < BITS; p++) {
+                const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[rb] + p * plane_stride + w));
+#pragma unroll
+                for (int i = 0; i < 4; i++) q[rb][p][i] = v[i];
+            }
+    };
+
+    // ---- activation stages: thread = (unit su of the 256-byte run, row sr + 16 i)
+    const int su = tid & 15, sr = tid >> 4;
+    const int full_chunks = W >> 5;
+    const uint32_t tail_stride = (uint32_t)(W & 31) * 16u;  // bytes of x between byte groups in the tail chunk
+    uint32_t xrow[MBW];                                     // byte offset of this thread's activation rows (past M: row M-1)
+#pragma unroll
+    for (int i = 0; i < MBW; i++) xrow[i] = (uint32_t)min(m0 + sr + 16 * i, M - 1) * (uint32_t)K * 2u;
+    // returns whether this thread's unit lies inside the row (the loaded bytes are some valid ones otherwise)
+    auto stage_load = [&](int step, int j, u32x4(&xr)[MBW]) {
+        const int w0 = 16 * step, chunk = w0 >> 5;
+        const bool valid = w0 + su < W;
+        const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)((w0 & 31) + (valid ? su : 0)) << 4) +
+                              (uint32_t)j * (chunk == full_chunks ? tail_stride : 512u);
+#pragma unroll
+        for (int i = 0; i < MBW; i++)
+            xr[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + (size_t)(xrow[i] + koff));
+        return valid;
+    };
+    // units of words past the row end hold zeros
+    auto stage_store = [&](int buf, const u32x4(&xr)[MBW], bool valid) {
+#pragma unroll
+        for (int i = 0; i < MBW; i++) xt[buf][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
+    };
+
+    // ---- prologue: planes of step 0, stage 0, tables
+    uint32_t q[RB][BITS][4];
+    fetch(step_at(0), q);
+    // stage t + 2 is requested while stage t is in work: slot t & 1 of xr carries stages t, t + 2, ...
+    u32x4 xr[2][MBW];
+    bool xvalid[2];
+    xvalid[0] = stage_load(step_at(0), 0, xr[0]);
+    if constexpr (PAIR) {
+        // each wave builds the pair tables of its own rows, eight rows' loads in flight at a time
+        const PairLane<BITS> pl = pair_lane<BITS>(lane);
+#pragma unroll
+        for (int r0 = 0; r0 < WROWS; r0 += 8) {
+            TableWords<BITS> tw[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) tw[i] = lookup_table_fetch<BITS>(lut + (size_t)min(n0 + r0 + i, N - 1) * NC, lane, pl);
+#pragma unroll
+            for (int i = 0; i < 8; i++) lookup_table_stage<BITS>(tw[i], &tables[wv * WROWS + r0 + i][0], lane);
+        }
+    } else {
+        // the tables of the workgroup's rows are contiguous in lut (rows past N re-read the last 16 bytes of the array)
+        constexpr int TQ = BN * NC / 8;  // 16-byte quads
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
+        u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[0][0]);
+        const long long first = (long long)nb * (NC / 8), last = (long long)N * (NC / 8) - 1;
+        for (int i = tid; i < TQ; i += NTHR) dst[i] = src[min(first + i, last)];
+    }
+    stage_store(0, xr[0], xvalid[0]);
+    xvalid[1] = stage_load(step_at(0), 1, xr[1]);  // every row has at least four stages
+    __syncthreads();
+
+    typedef __attribute__((address_space(3))) uint16_t lds_u16_t;
+    typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
+    const uint32_t tab_base0 =
+        (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t *)&tables[0][0]) + (uint32_t)(wv * WROWS + col) * TB;
+
+    float4_t acc[RB][MBW];
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+        for (int mb = 0; mb < MBW; mb++) acc[rb][mb] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    constexpr int PRE = BITS <= 7 ? 1 : 0;  // index bytes hold the byte offset into the table where that fits a byte
+    constexpr int NRAW = PAIR ? 4 : 8;      // table reads per B operand
+    uint32_t idx[4][RB][NRAW];              // indices of the 16 words of the step (lane: words 16 step + 4 wi + grp)
+    half8_t afrag[2][MBW];                  // A operands of the octet in work and of the next one
+    uint32_t braw[2][RB][NRAW];             // table entries of their B operands as they come from LDS
+    // A operands of octet wi of the stage in buffer buf
+    auto issue_a = [&](auto buf_c, auto wi_c, half8_t(&a)[MBW]) {
+        constexpr int buf = decltype(buf_c)::value, wi = decltype(wi_c)::value;
+#pragma unroll
+        for (int mb = 0; mb < MBW; mb++) a[mb] = __builtin_bit_cast(half8_t, xt[buf][mb * 16 + col][(4 * wi + grp) ^ col]);
+    };
+    // table reads for the eight weights of byte group j of word wi of each row block
+    auto issue_b = [&](auto j_c, auto wi_c, uint32_t(&raw)[RB][NRAW]) {
+        constexpr int c = 3 - decltype(j_c)::value, wi = decltype(wi_c)::value;
+        static_for<RB>([&](auto rb_c) {
+            constexpr int rb = decltype(rb_c)::value;
+            const uint32_t tab_base = tab_base0 + rb * (kGemmRows * TB);
+            static_for<NRAW>([&](auto e_c) {
+                constexpr int i = decltype(e_c)::value;
+                if constexpr (PAIR) {
+                    raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(byte_add<c>(tab_base, idx[wi][rb][i]));
+                } else {
+                    uint32_t a0;
+                    if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
+                    else a0 = tab_base + byte_offset<c, 1>(idx[wi][rb][i]);
+                    raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(a0);
+                }
+            });
+        });
+    };
+    // words past the row end: zero weights (their activations are zeros too)
+    auto finish_b = [&](const uint32_t(&raw)[RB][NRAW], bool alive, half8_t(&b)[RB]) {
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+            u32x4 bw;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t packed;
+                if constexpr (PAIR) packed = raw[rb][i];
+                else packed = raw[rb][2 * i] | (raw[rb][2 * i + 1] << 16);
+                bw[i] = alive ? packed : 0u;
+            }
+            b[rb] = __builtin_bit_cast(half8_t, bw);
+        }
+    };
+    for (int it = 0; it < steps; it++) {
+        const int step = step_at(it), step_next = step_at(it + 1);
+        const bool last = it + 1 == steps;
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++) {
+#pragma unroll
+            for (int p = 0; p < BITS; p++) transpose_rows4(q[rb][p]);
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++) {
+                uint32_t qq[BITS];
+#pragma unroll
+                for (int p = 0; p < BITS; p++) qq[p] = q[rb][p][wi];
+                if constexpr (PAIR) planes_to_adjacent_pairs<BITS>(qq, idx[wi][rb]);
+                else planes_to_indices<BITS, PRE>(qq, idx[wi][rb]);
+            }
+        }
+        if (!last) fetch(step_next, q);
+        const bool partial = 16 * (step + 1) > W;
+        bool live[4];
+#pragma unroll
+        for (int wi = 0; wi < 4; wi++) live[wi] = !partial || 16 * step + 4 * wi + grp < W;
+
+        // One stage = byte group j of the 16 words: four octets (wi), each RB B operands and MBW A operands feeding
+        // RB x MBW matrix instructions.  The LDS reads of octet wi + 1 (A operands, table entries) are issued before
+        // the matrix instructions of octet wi; scheduling fences pin that order.  The table reads of the first octet
+        // of the next stage pass the barrier as well (the tables do not change).  Requesting the operands of a whole
+        // stage at once measured no faster: the LDS port, not its latency, bounds the stage (per stage and CU 4 x 4 x
+        // MBW KB of A operands and 4 x 4 x RB x 4..8 table reads against 4 x RB x MBW matrix instructions per wave).
+        static_for<4>([&](auto j_c) {
+            constexpr int j = decltype(j_c)::value, buf = j & 1;
+            const bool more = j < 3 || !last;     // a stage follows
+            const bool more2 = j < 2 || !last;    // two do
+            if (more2) xvalid[buf] = stage_load(j < 2 ? step : step_next, (j + 2) & 3, xr[buf]);
+            issue_a(std::integral_constant<int, buf>{}, std::integral_constant<int, 0>{}, afrag[0]);
+            if constexpr (j == 0) issue_b(j_c, std::integral_constant<int, 0>{}, braw[0]);
+            static_for<4>([&](auto wi_c) {
+                constexpr int wi = decltype(wi_c)::value, cur = wi & 1, nxt = cur ^ 1;
+                half8_t bfrag[RB];
+                finish_b(braw[cur], live[wi], bfrag);
+                if constexpr (wi < 3) {
+                    issue_a(std::integral_constant<int, buf>{}, std::integral_constant<int, wi + 1>{}, afrag[nxt]);
+                    issue_b(j_c, std::integral_constant<int, wi + 1>{}, braw[nxt]);
+                } else if constexpr (j < 3) {
+                    issue_b(std::integral_constant<int, j + 1>{}, std::integral_constant<int, 0>{}, braw[nxt]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int mb = 0; mb < MBW; mb++)
+#pragma unroll
+                    for (int rb = 0; rb < RB; rb++)
+                        acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[cur][mb], bfrag[rb], acc[rb][mb], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if (more) stage_store(buf ^ 1, xr[buf ^ 1], xvalid[buf ^ 1]);
+            // everyone is done with `buf`, and the other buffer is complete
+            lds_only_barrier();
+        });
+    }
+
+    // D[i][j]: lane l holds activation rows i = 4 (l / 16) + v of the block and weight row j = l % 16
+#pragma unroll
+    for (int rb = 0; rb < RB; rb++) {
+        const int n = n0 + rb * kGemmRows + col;
+#pragma unroll
+        for (int mb = 0; mb < MBW; mb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int m = m0 + mb * 16 + 4 * grp + v;
+                if (m < M && n < N) out[(size_t)m * N + n] = (half_t)acc[rb][mb][v];
+            }
+    }
+}
+
+}  // namespace ap

@@ -1,0 +1,28 @@
+// Tiled fused GEMM kernels of one bit-width (compile with -DAP_BITS=3..8) and their launch dispatch.
+#include "ap_gemmt.hpp"
+#include "ap_gemmt_launch.hpp"
+
+#ifndef AP_BITS
+#error "compile with -DAP_BITS=<3..8>"
+#endif
+
+namespace ap {
+
+template <int BITS>
+void launch_gemmt(const GemmtGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
+                  uint16_t *out, int M, int N, int K, hipStream_t stream) {
+    const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
+    half_t *oh = reinterpret_cast<half_t *>(out);
+    const dim3 block(kWave, kGemmtWaves), grid(geo.grid_n, geo.grid_m);
+    // one block of 16 weight rows per wave: two measured slower on every shape (a quarter of the workgroups, and the
+    // LDS traffic per matrix instruction falls by less than a third)
+    if (geo.mbw == 8)
+        gemmt_kbit_kernel<BITS, 1, 8><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+    else
+        gemmt_kbit_kernel<BITS, 1, 4><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+}
+
+template void launch_gemmt<AP_BITS>(const GemmtGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *,
+                                    int, int, int, hipStream_t);
+
+}  // namespace ap

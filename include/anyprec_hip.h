@@ -88,11 +88,14 @@ int ap_matmul_kbit_swiglu(const uint16_t *x, const uint32_t *qweight_gate, const
 /* Fused dequant -> MFMA GEMM, M >= 1: out[M,N] = x[M,K] . dequant(qweight, lut)^T
  * without materialising the fp16 weight.  No single counterpart in the reference: it is the
  * M > 8 branch of AnyPrecisionLinear.forward (AnyPrecisionLinear.py:60-62: dequant_kbit,
- * main.cu:60-91, then torch.matmul) fused.  One launch serves up to 128 activation rows (more
- * than 32 may run as launches of 32 rows each); beyond 128 the call issues one launch per 128
- * rows, in order, on the same stream, re-reading the planes for each -- correct for every M, but
- * from a few hundred rows on dequant + a library GEMM is the faster pair.  fp32 accumulation,
- * fp16 result. */
+ * main.cu:60-91, then torch.matmul) fused.  Two kernels: up to 128 activation rows a K-split
+ * kernel with the weights of 16 rows in registers (more than 32 rows may run as launches of 32
+ * each); beyond 128 rows, and from 48..96 rows on where it measured faster, a tiled kernel whose
+ * workgroups own 64 weight rows x 64 or 128 activation rows for the whole of K, ONE launch for any
+ * M (it needs K % 128 == 0; other row lengths go through the K-split kernel in chunks of 128 rows,
+ * in order, on the same stream).  Correct for every M; faster than dequant + a library GEMM up to
+ * about 256 rows at 3 bits and 64..128 rows at more bits -- beyond that use that pair.
+ * fp32 accumulation, fp16 result. */
 int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int M, int N, int K, int w_bits, void *stream);
 
@@ -130,7 +133,8 @@ int ap_matmul_kbit_group_route(int count, const int *N, int M, int K, int w_bits
  * beyond the 1e-2 bar of the entry points; the defaults are what measured fastest.  Names:
  * gemv_target_waves, gemv_rows, gemv_wpl, dequant_blocks_per_cu, matmul_mfma_from, gemm_split,
  * matmul_mfma4, gemv4_groups, gemm_rb2, gemv_stream, gemv_stream_waves, gemv_fine,
- * gemv_persist, gemv_persist_waves, gemm_walk, gemm_walk_wgs.  Returns AP_OK, AP_ENULL or AP_EKNOB. */
+ * gemv_persist, gemv_persist_waves, gemm_walk, gemm_walk_wgs, gemm_tiled, gemm_tile.  Returns AP_OK, AP_ENULL
+ * or AP_EKNOB. */
 int ap_set_tuning(const char *name, int value);
 int ap_get_tuning(const char *name, int *value);
 

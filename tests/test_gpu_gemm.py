@@ -194,3 +194,74 @@ def test_row_walking_kernel_on_a_wide_linear_by_default(ext, oracle):
         got = ext.gemm_kbit(xg, q, luts[b], b)
         _, want = oracle.matmul_kbit(x, L.qweight[:, rows], L.luts[b][rows], b, return_f64=True)
         assert_close_gemv(got[:, torch.from_numpy(rows).cuda()], want, f"N={N} K={K} b={b} M={M}")
+
+
+def test_tiled_kernel_agrees_with_the_oracle(ext, oracle):
+    """The tiled kernel (a workgroup owns 64 weight rows x 64 or 128 activation rows for the whole of K, activations
+    staged once per workgroup in LDS) forced with gemm_tiled = 2 and both tiles, on shapes small enough for the oracle:
+    ragged row counts on both sides, one stage per byte group (K = 128), a tail chunk with a partial last step
+    (K = 2176, 11008), several tiles of activation rows (M = 300).  Every output sums its products in the same order
+    whatever the tile, so the two tiles agree bit for bit."""
+    from any_precision_amd import _capi
+    for N, K in ((200, 128), (64, 1024), (130, 2176), (96, 11008), (257, 4096)):
+        L = make(N, K, seed=N + K)
+        q, luts = layer_to_gpu(L)
+        for b in range(3, 9):
+            for M in (1, 17, 64, 65, 130, 300):
+                print(f"tiled N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                with _capi.tuning(gemm_tiled=2, gemm_tile=4):
+                    small = ext.gemm_kbit(xg, q, luts[b], b)
+                with _capi.tuning(gemm_tiled=2, gemm_tile=8):
+                    large = ext.gemm_kbit(xg, q, luts[b], b)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                assert_close_gemv(small, want, f"tiled N={N} K={K} b={b} M={M}")
+                assert torch.equal(small.view(torch.int16), large.view(torch.int16)), (N, K, b, M)
+    # one-hot activation rows return columns of the dequantised weight exactly (K = 2176: also the partial step)
+    N, K = 130, 2176
+    L = make(N, K, seed=N + K)
+    q, luts = layer_to_gpu(L)
+    ks = [0, 7, 8, 255, 256, 1023, 1024, 2047, 2048, 2079, 2080, 2111, 2112, 2143, 2144, 2175, 31, 32, 1500, 100] * 4
+    x = torch.zeros((len(ks), K), dtype=torch.float16, device="cuda")
+    for m, k in enumerate(ks):
+        x[m, k] = 1.0
+    for b in (3, 5, 8):
+        w = oracle.dequant_kbit(L.qweight, L.luts[b], b)
+        with _capi.tuning(gemm_tiled=2):
+            got = ext.gemm_kbit(x, q, luts[b], b)
+        for m, k in enumerate(ks):
+            assert_bit_exact(got[m], w[:, k], f"tiled one-hot b={b} k={k}")
+
+
+def test_tiled_kernel_by_default_beyond_128_rows(ext, oracle):
+    """More than 128 activation rows on rows of a multiple of 128 elements take the tiled kernel by the default rule
+    (other row lengths go in chunks of 128 through the K-split kernel): against the oracle, equal to the forced tiled
+    launch bit for bit, and the same from a replayed HIP graph."""
+    from any_precision_amd import _capi
+    N, K = 176, 4096
+    L = make(N, K, seed=11)
+    q, luts = layer_to_gpu(L)
+    for b, M in ((3, 129), (4, 200), (8, 300)):
+        print(f"tiled default b={b} M={M}", flush=True)
+        x, xg = _x(M, K, seed=M)
+        got = ext.gemm_kbit(xg, q, luts[b], b)
+        _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+        assert_close_gemv(got, want, f"tiled default b={b} M={M}")
+        with _capi.tuning(gemm_tiled=2):
+            forced = ext.gemm_kbit(xg, q, luts[b], b)
+        assert torch.equal(got.view(torch.int16), forced.view(torch.int16))
+        with _capi.tuning(gemm_tiled=0):
+            chunks = ext.gemm_kbit(xg, q, luts[b], b)
+        assert_close_gemv(chunks, want, f"chunks b={b} M={M}")
+        out = torch.zeros((M, N), dtype=torch.float16, device="cuda")
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            rc = _capi.lib.ap_gemm_kbit(xg.data_ptr(), q.data_ptr(), luts[b].data_ptr(), out.data_ptr(), M, N, K, b,
+                                        torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+        for rep in range(3):
+            out.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out.view(torch.int16), got.view(torch.int16)), rep
