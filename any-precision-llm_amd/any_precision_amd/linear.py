@@ -25,18 +25,21 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     up to 64 on linears of fewer than 8192 rows, and on larger ones at up to 5 bits -- except, on rows of more
     than 4096 elements, from 6 bits on linears of 5120 rows or more (5120 x 13824, 8 bits: 121 us against 86)
     and from 5 bits on linears of at most 2048 rows (1024 x 8192); up to 128 on linears of 4096..8191
-    rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).  With the tiled kernel (rows of a multiple of
-    128 elements, linears of at least 4096 rows): at 3 bits up to 256 activation rows everywhere (4096 x 4096: 26 us
-    against 39-51; 11008 x 4096: 40-57 against 57-73; 8192 x 8192: 53-79 against 82-113), at 4 bits up to 128 on rows
-    of at most 8192 elements (11008 x 4096: 52 against 57-59) and up to 256 on linears of fewer than 8192 rows of at
-    most 5120 elements (4096 x 4096: 38 against 40-51).  Beyond, one table lookup per weight and tile of activation
-    rows costs more than materialising the weight once."""
+    rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).
+    With the tiled kernel (rows of a multiple of 128 elements, linears of at least 4096 rows): at 3 bits up to 256
+    activation rows everywhere (4096 x 4096: 24-25 us against 39-43; 11008 x 4096: 48-71 against 58-73; 4096 x 11008:
+    63-65 against 78-84); at 4 bits up to 128 (11008 x 4096: 52 against 57; 4096 x 11008: 77 against 85); at 4 and 5
+    bits up to 256 on linears of fewer than 8192 rows of at most 4096 elements (4096 x 4096: 30-35 against 40-44); and
+    up to 64 rows at every bit-width on linears of 8192 rows or more of at most 4096 elements (11008 x 4096, 8 bits:
+    41 against 53).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising
+    the weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
-    if GEMM_MAX_M and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
-        if w_bits == 3:
+    if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
+        small = out_features < 8192 and in_features <= 4096
+        if w_bits == 3 or (w_bits == 4 and rows <= 128) or (w_bits <= 5 and small):
             return True
-        if w_bits == 4 and ((rows <= 128 and 0 < in_features <= 8192) or (out_features < 8192 and 0 < in_features <= 5120)):
+        if rows <= 64 and out_features >= 8192 and in_features <= 4096:
             return True
     if rows <= min(64, GEMM_MAX_M):
         if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):

@@ -46,6 +46,7 @@ enum {
     kGemmWalkWgs,       // workgroups per CU its grid aims for
     kGemmTiled,         // tiled fused GEMM (ap_gemm_kbit): 0 never, 1 where it pays, 2 wherever it fits
     kGemmTile,          // > 0: blocks of 16 activation rows in its tile, 4 or 8
+    kGemmTileSplit,     // > 0: groups of four waves per workgroup of the 64-row tile, each on its share of K: 1 or 2
     kKnobCount
 };
 Knob g_knobs[kKnobCount] = {
@@ -54,6 +55,7 @@ Knob g_knobs[kKnobCount] = {
     {"gemm_rb2", 1},              {"gemv_stream", 1},    {"gemv_stream_waves", 24},
     {"gemv_fine", 1},             {"gemv_persist", 1},   {"gemv_persist_waves", 8},
     {"gemm_walk", 1},             {"gemm_walk_wgs", 1},  {"gemm_tiled", 1},   {"gemm_tile", 0},
+    {"gemm_tile_split", 0},
 };
 inline int knob(int k) { return __atomic_load_n(&g_knobs[k].value, __ATOMIC_RELAXED); }
 
@@ -391,32 +393,38 @@ bool gemmw_geometry(int M, int N, int K, int w_bits, GemmwGeometry *geo) {
 
 // Tile of the tiled fused GEMM (ap_gemmt.hpp) for a shape; false if the kernel does not serve it.  64 weight rows x
 // 64 activation rows unless that makes several workgroups per CU: then 64 x 128, which halves the table lookups per
-// matrix instruction (measured on 4096 x 4096, 11008 / 14336 x 4096, 4096 x 11008, 5120 x 5120, 8192 x 8192 at 48..384
+// matrix instruction (measured on 4096 x 4096, 11008 / 14336 x 4096, 4096 x 11008, 5120 x 5120, 8192 x 8192 at 48..512
 // rows: the larger tile wins from about 3 workgroups of the smaller one per CU on at 3 bits, from 1.3 on at 4+ bits).
+// Grids of at most one small tile per CU run it with two groups of waves, each on half of K (4096 x 4096 at 128..256
+// rows: 30 us against 37 at 4 bits, 38 against 50 at 8; 4096 x 11008: 77 against 100 at 4 bits); with more tiles than
+// CUs the second group only takes LDS from the next workgroup (11008 x 4096, 256 rows, 3 bits: 71 us against 56).
 bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
     if ((K & 127) != 0 || (long long)M * K * 2 > 0xffffffffLL) return false;
-    const int forced = knob(kGemmTile);
+    const int forced = knob(kGemmTile), force_kh = knob(kGemmTileSplit);
+    const long long small = (long long)((N + 63) / 64) * ((M + 63) / 64);  // tiles of 64 x 64
     int mbw = 4;
     if (forced > 0) {
         if (forced != 4 && forced != 8) return false;
         mbw = forced;
     } else if (M > 64) {
-        const long long small = (long long)((N + 63) / 64) * ((M + 63) / 64);
         if (10 * small >= (w_bits == 3 ? 30LL : 13LL) * cu_count()) mbw = 8;
     }
     geo->mbw = mbw;
+    // two K halves need at least two steps of 512 elements
+    geo->kh = mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && small <= cu_count())) ? 2 : 1;
     geo->grid_n = (N + 63) / 64;
     geo->grid_m = (M + 16 * mbw - 1) / (16 * mbw);
     return geo->grid_m <= 65535;
 }
 
 // Where the tiled kernel is the fastest fused form (same sweep, against the K-split kernel, which serves more than 128
-// rows in chunks of 128): always beyond 128 rows; at 3 bits from 96 rows on, from 48 on linears of at least 8192 rows of
-// at most 4096 elements (11008 x 4096 at 64 rows: 27 us against 38); at 4..8 bits from 64 rows on such linears only.
+// rows in chunks of 128): always beyond 128 rows; on linears of at least 8192 rows of at most 4096 elements from 64
+// rows on (11008 x 4096 at 64 rows: 26-41 us against 38-58), at 3 bits from 48; elsewhere at 3 bits from 96 rows on and
+// at 4 and 5 bits from 120 (4096 x 4096 at 128 rows: 30 / 33 us against 34 / 35; 4096 x 11008: 77 / 84 against 88 / 98).
 bool gemmt_pays(int M, int N, int K, int w_bits) {
     if (M > 128) return true;
-    const bool wide = N >= 8192 && K <= 4096;
-    return w_bits == 3 ? M >= (wide ? 48 : 96) : (wide && M >= 64);
+    if (N >= 8192 && K <= 4096) return M >= (w_bits == 3 ? 48 : 64);
+    return w_bits == 3 ? M >= 96 : (w_bits <= 5 && M >= 120);
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).

@@ -25,8 +25,12 @@
 
 namespace ap {
 
-template <int BITS, int RB, int MBW>
-__global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
+// KH = 1 or 2 groups of four waves per workgroup; with 2, group kh walks half of K (steps kh * ceil(steps / 2) ..) on its
+// own stage buffers and the two partial tiles are added in LDS at the end (group 0's sum + group 1's, always in that
+// order).  Twice the waves per tile: for grids that leave CUs with one workgroup of four waves, where no pipe is busy
+// and waves wait for each other's LDS round trips.
+template <int BITS, int RB, int MBW, int KH>
+__global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K) {
     constexpr int NC = 1 << BITS;
@@ -38,11 +42,14 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
     constexpr int BN = kGemmtWaves * WROWS, BM = 16 * MBW;
     constexpr int NTHR = kGemmtWaves * kWave;
     __shared__ __attribute__((aligned(16))) uint8_t tables[BN][TB];
-    __shared__ u32x4 xt[2][BM][16];  // [stage buffer][activation row][16-byte unit ^ (row & 15)]
+    __shared__ u32x4 xt[KH][2][BM][16];  // [K half][stage buffer][activation row][16-byte unit ^ (row & 15)]
+    static_assert(KH == 1 || KH == 2, "");
+    static_assert(KH == 1 || RB * MBW * 4 * kWave * kGemmtWaves * 4 <= (int)sizeof(xt) / KH, "partial tiles fit a half's stage buffers");
 
     const int lane = threadIdx.x;
-    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.y);
-    const int tid = wv * kWave + lane;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int wv = wave % kGemmtWaves, kh = wave / kGemmtWaves;  // row group of the wave, its half of K
+    const int tid = wv * kWave + lane;                            // thread within the half
     const int col = lane & 15, grp = lane >> 4;
     const int W = K >> 5;
     const size_t plane_stride = (size_t)N * W;
@@ -50,9 +57,12 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
     const int n0 = nb + wv * WROWS;     // ... of this wave
     const int m0 = blockIdx.y * BM;     // first activation row of the tile
     const int steps = (W + 15) >> 4;    // 16 words of every row per step
+    const int nit = (steps + KH - 1) / KH;   // steps per K half; a half with one step fewer idles through the last
     // (all workgroups walk K in the same order: those in flight then read the same columns of the activations at
     // about the same time and share them in L2 -- walking from staggered starting steps measured 10-35 % slower)
-    auto step_at = [&](int i) { return i < steps ? i : 0; };
+    // Iteration i of this half: its step, clamped into the row (an idle iteration loads valid bytes and uses none).
+    auto step_at = [&](int i) { return min(kh * nit + i, steps - 1); };
+    auto active_at = [&](int i) { return kh * nit + i < steps; };
 
     const uint32_t *wrow[RB];  // rows past N repeat row N-1 and are not stored
 #pragma unroll
@@ -79,9 +89,9 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
 #pragma unroll
     for (int i = 0; i < MBW; i++) xrow[i] = (uint32_t)min(m0 + sr + 16 * i, M - 1) * (uint32_t)K * 2u;
     // returns whether this thread's unit lies inside the row (the loaded bytes are some valid ones otherwise)
-    auto stage_load = [&](int step, int j, u32x4(&xr)[MBW]) {
+    auto stage_load = [&](int step, bool active, int j, u32x4(&xr)[MBW]) {
         const int w0 = 16 * step, chunk = w0 >> 5;
-        const bool valid = w0 + su < W;
+        const bool valid = active && w0 + su < W;
         const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)((w0 & 31) + (valid ? su : 0)) << 4) +
                               (uint32_t)j * (chunk == full_chunks ? tail_stride : 512u);
 #pragma unroll
@@ -92,7 +102,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
     // units of words past the row end hold zeros
     auto stage_store = [&](int buf, const u32x4(&xr)[MBW], bool valid) {
 #pragma unroll
-        for (int i = 0; i < MBW; i++) xt[buf][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
+        for (int i = 0; i < MBW; i++) xt[kh][buf][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
     };
 
     // ---- prologue: planes of step 0, stage 0, tables
@@ -101,17 +111,19 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
     // stage t + 2 is requested while stage t is in work: slot t & 1 of xr carries stages t, t + 2, ...
     u32x4 xr[2][MBW];
     bool xvalid[2];
-    xvalid[0] = stage_load(step_at(0), 0, xr[0]);
+    xvalid[0] = stage_load(step_at(0), active_at(0), 0, xr[0]);
     if constexpr (PAIR) {
-        // each wave builds the pair tables of its own rows, eight rows' loads in flight at a time
+        // each wave builds pair tables of its own rows (with two K halves: its half of them), eight rows' loads in
+        // flight at a time
         const PairLane<BITS> pl = pair_lane<BITS>(lane);
 #pragma unroll
-        for (int r0 = 0; r0 < WROWS; r0 += 8) {
+        for (int r0 = 0; r0 < WROWS / KH; r0 += 8) {
+            const int r1 = kh * (WROWS / KH) + r0;
             TableWords<BITS> tw[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) tw[i] = lookup_table_fetch<BITS>(lut + (size_t)min(n0 + r0 + i, N - 1) * NC, lane, pl);
+            for (int i = 0; i < 8; i++) tw[i] = lookup_table_fetch<BITS>(lut + (size_t)min(n0 + r1 + i, N - 1) * NC, lane, pl);
 #pragma unroll
-            for (int i = 0; i < 8; i++) lookup_table_stage<BITS>(tw[i], &tables[wv * WROWS + r0 + i][0], lane);
+            for (int i = 0; i < 8; i++) lookup_table_stage<BITS>(tw[i], &tables[wv * WROWS + r1 + i][0], lane);
         }
     } else {
         // the tables of the workgroup's rows are contiguous in lut (rows past N re-read the last 16 bytes of the array)
@@ -119,10 +131,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
         const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
         u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[0][0]);
         const long long first = (long long)nb * (NC / 8), last = (long long)N * (NC / 8) - 1;
-        for (int i = tid; i < TQ; i += NTHR) dst[i] = src[min(first + i, last)];
+        for (int i = kh * NTHR + tid; i < TQ; i += KH * NTHR) dst[i] = src[min(first + i, last)];
     }
     stage_store(0, xr[0], xvalid[0]);
-    xvalid[1] = stage_load(step_at(0), 1, xr[1]);  // every row has at least four stages
+    xvalid[1] = stage_load(step_at(0), active_at(0), 1, xr[1]);  // every row has at least four stages
     __syncthreads();
 
     typedef __attribute__((address_space(3))) uint16_t lds_u16_t;
@@ -145,7 +157,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
     auto issue_a = [&](auto buf_c, auto wi_c, half8_t(&a)[MBW]) {
         constexpr int buf = decltype(buf_c)::value, wi = decltype(wi_c)::value;
 #pragma unroll
-        for (int mb = 0; mb < MBW; mb++) a[mb] = __builtin_bit_cast(half8_t, xt[buf][mb * 16 + col][(4 * wi + grp) ^ col]);
+        for (int mb = 0; mb < MBW; mb++) a[mb] = __builtin_bit_cast(half8_t, xt[kh][buf][mb * 16 + col][(4 * wi + grp) ^ col]);
     };
     // table reads for the eight weights of byte group j of word wi of each row block
     auto issue_b = [&](auto j_c, auto wi_c, uint32_t(&raw)[RB][NRAW]) {
@@ -181,9 +193,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
             b[rb] = __builtin_bit_cast(half8_t, bw);
         }
     };
-    for (int it = 0; it < steps; it++) {
+    for (int it = 0; it < nit; it++) {
         const int step = step_at(it), step_next = step_at(it + 1);
-        const bool last = it + 1 == steps;
+        const bool active = active_at(it), active_next = active_at(it + 1);
+        const bool last = it + 1 == nit;
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
 #pragma unroll
@@ -201,7 +214,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
         const bool partial = 16 * (step + 1) > W;
         bool live[4];
 #pragma unroll
-        for (int wi = 0; wi < 4; wi++) live[wi] = !partial || 16 * step + 4 * wi + grp < W;
+        for (int wi = 0; wi < 4; wi++) live[wi] = active && (!partial || 16 * step + 4 * wi + grp < W);
 
         // One stage = byte group j of the 16 words: four octets (wi), each RB B operands and MBW A operands feeding
         // RB x MBW matrix instructions.  The LDS reads of octet wi + 1 (A operands, table entries) are issued before
@@ -213,7 +226,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
             constexpr int j = decltype(j_c)::value, buf = j & 1;
             const bool more = j < 3 || !last;     // a stage follows
             const bool more2 = j < 2 || !last;    // two do
-            if (more2) xvalid[buf] = stage_load(j < 2 ? step : step_next, (j + 2) & 3, xr[buf]);
+            if (more2) xvalid[buf] = stage_load(j < 2 ? step : step_next, j < 2 ? active : active_next, (j + 2) & 3, xr[buf]);
             issue_a(std::integral_constant<int, buf>{}, std::integral_constant<int, 0>{}, afrag[0]);
             if constexpr (j == 0) issue_b(j_c, std::integral_constant<int, 0>{}, braw[0]);
             static_for<4>([&](auto wi_c) {
@@ -241,6 +254,27 @@ __global__ __launch_bounds__(kGemmtWaves *kWave) void gemmt_kbit_kernel(
     }
 
     // D[i][j]: lane l holds activation rows i = 4 (l / 16) + v of the block and weight row j = l % 16
+    if constexpr (KH == 2) {
+        // the last barrier of the loop has passed: nobody reads the stage buffers any more.  Group 1 parks its tiles in
+        // its own buffers, group 0 adds them to its own.
+        float *park = reinterpret_cast<float *>(&xt[1][0][0][0]) + wv * (RB * MBW * 4 * kWave);
+        if (kh == 1) {
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+                for (int mb = 0; mb < MBW; mb++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) park[((rb * MBW + mb) * 4 + v) * kWave + lane] = acc[rb][mb][v];
+        }
+        __syncthreads();
+        if (kh == 1) return;
+#pragma unroll
+        for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+            for (int mb = 0; mb < MBW; mb++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[rb][mb][v] += park[((rb * MBW + mb) * 4 + v) * kWave + lane];
+    }
 #pragma unroll
     for (int rb = 0; rb < RB; rb++) {
         const int n = n0 + rb * kGemmRows + col;

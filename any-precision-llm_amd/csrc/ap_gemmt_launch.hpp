@@ -10,11 +10,12 @@ constexpr int kGemmtWaves = 4;  // waves per workgroup, each on its own block(s)
 
 struct GemmtGeometry {
     int mbw;     // blocks of 16 activation rows per workgroup tile (4 or 8); a workgroup owns 64 weight rows
+    int kh;      // groups of four waves per workgroup, each on its share of K (1, or 2 with mbw = 4)
     int grid_n;  // ceil(N / 64)
     int grid_m;  // ceil(M / (16 mbw))
 };
 
-// Launches gemmt_kbit_kernel<BITS, 1, geo.mbw> on `stream`.  K must be a multiple of 128.
+// Launches gemmt_kbit_kernel<BITS, 1, geo.mbw, geo.kh> on `stream`.  K must be a multiple of 128.
 template <int BITS>
 void launch_gemmt(const GemmtGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                   uint16_t *out, int M, int N, int K, hipStream_t stream);

@@ -34,7 +34,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--workload", default="llama2_7b_layer_batch1",
                     choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model",
-                             "llama2_7b_decode", "llama2_7b_prefill", "gemv_kernel_variants", "routing_audit"),
+                             "llama2_7b_decode", "llama2_7b_prefill", "llama2_7b_gemm_rows", "gemv_kernel_variants",
+                             "routing_audit"),
                     help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
                          "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
                          "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.  "
@@ -42,6 +43,9 @@ def parse_args():
                          "256 tokens after a 128-token prompt, per w_bits.  "
                          "llama2_7b_prefill: the seven linears of a layer on 32 x 512 = 16384 activation rows "
                          "(dequant_kbit + library GEMM, the large-batch branch of AnyPrecisionLinear).  "
+                         "llama2_7b_gemm_rows: ap_gemm_kbit on the three linear shapes of the layer at 64..512 activation "
+                         "rows: its default launch, the K-split and the tiled kernel forced, dequant_kbit + library GEMM "
+                         "beside them; with --eager one launch of the tiled kernel per case only (for counter runs).  "
                          "gemv_kernel_variants: the four dot-product GEMV kernels forced in turn (tuning knobs) on "
                          "the headline shapes and on 28672 x 8192, batch 1, beside the read-only stream; with "
                          "--eager the launches go out one by one (the form rocprofv3 counter runs need).  "
@@ -112,6 +116,8 @@ def main():
         return gemv_kernel_variants(args, torch, _capi, synth)
     if args.workload == "routing_audit":
         return routing_audit(args, torch, _capi, synth)
+    if args.workload == "llama2_7b_gemm_rows":
+        return gemm_rows(args, torch, _capi, synth)
     if args.workload == "llama2_7b_decode":
         with torch.inference_mode():     # the decoder captures its graphs in inference mode; stay in it
             return decode_tokens(args, torch, _capi, synth)
@@ -871,6 +877,69 @@ def routing_audit(args, torch, _capi, synth):
                                + "; cold weight sets; HIP graphs; alternatives forced through ap_set_tuning"},
         "cases": len(cases), "worst_excess": max((l["excess"] for l in losses), default=0.0),
         "losses": sorted(losses, key=lambda l: -l["excess"]), "all_cases": cases}))
+
+
+def gemm_rows(args, torch, _capi, synth):
+    """ap_gemm_kbit at 64..512 activation rows on 4096 x 4096, 11008 x 4096, 4096 x 11008 (cold weight sets, HIP graphs):
+    the default launch, the K-split kernel (chunks of 128 rows beyond 128), the tiled kernel with either tile, and
+    dequant_kbit + torch.matmul, which is what AnyPrecisionLinear falls back to."""
+    import any_precision_ext as ext
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    side = torch.cuda.Stream()
+    bits, Ms = (3, 4, 5, 8), (64, 128, 256, 512)
+    cases = []
+    for N, K in ((4096, 4096), (11008, 4096), (4096, 11008)):
+        P = WeightPool(torch, N, K, max(4, int(args.pool_gb * 1e9 / (N * K)) + 1), gen, bits=bits)
+        cur = {"j": 0}
+        for b in bits:
+            for M in Ms:
+                x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+                out = torch.empty((M, N), dtype=torch.float16, device="cuda")
+
+                def fused(st):
+                    cur["j"] = (cur["j"] + 1) % P.sets
+                    rc = lib.ap_gemm_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                          out.data_ptr(), M, N, K, b, st)
+                    if rc != 0:
+                        raise RuntimeError(_capi.strerror(rc))
+
+                def pair(st):
+                    cur["j"] = (cur["j"] + 1) % P.sets
+                    torch.matmul(x, ext.dequant_kbit(P.qweight[cur["j"]], P.luts[b][cur["j"]], b).T, out=out)
+
+                if args.eager:
+                    with _capi.tuning(gemm_tiled=2):
+                        fused(torch.cuda.current_stream().cuda_stream)
+                    torch.cuda.synchronize()
+                    continue
+                reps = min(P.sets, 12)
+                us = {"default": _graph_us(torch, side, fused, reps), "dequant_matmul": _graph_us(torch, side, pair, reps)}
+                for name, knobs in (("k_split", {"gemm_tiled": 0}), ("tiled_64", {"gemm_tiled": 2, "gemm_tile": 4}),
+                                    ("tiled_128", {"gemm_tiled": 2, "gemm_tile": 8})):
+                    with _capi.tuning(**knobs):
+                        us[name] = _graph_us(torch, side, fused, reps)
+                fastest = min(us[k] for k in us if k not in ("default", "dequant_matmul"))
+                cases.append(dict({"N": N, "K": K, "w_bits": b, "M": M}, **{k + "_us": round(v, 1) for k, v in us.items()},
+                                  default_TFLOPs=round(2.0 * M * N * K / us["default"] / 1e6, 1),
+                                  default_over_fastest_fused=round(us["default"] / fastest, 3),
+                                  fused_over_dequant_matmul=round(us["default"] / us["dequant_matmul"], 3)))
+        del P
+        torch.cuda.empty_cache()
+    if args.eager:
+        print(json.dumps({"metric": "one eager launch of the tiled fused GEMM per (shape, w_bits, rows)", "value": None,
+                          "unit": "", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None, "data": "synthetic",
+                          "config": {"workload": "llama2_7b_gemm_rows --eager"}}))
+        return
+    wins = [c for c in cases if c["fused_over_dequant_matmul"] < 1.0]
+    print(json.dumps({
+        "metric": "share of (shape, w_bits, rows) cases where ap_gemm_kbit's default launch beats dequant_kbit + library GEMM",
+        "value": round(len(wins) / len(cases), 4), "unit": "fraction", "n_gpus": 1, "higher_is_better": True,
+        "vs_baseline": None, "data": "synthetic", "dtype": "fp16 operands, u32 bitplanes, fp32 accumulate",
+        "config": {"workload": "ap_gemm_kbit on 4096x4096, 11008x4096, 4096x11008 at 64, 128, 256, 512 activation rows, "
+                               "w_bits 3, 4, 5, 8; cold weight sets; HIP graphs"},
+        "worst_default_over_fastest_fused": max(c["default_over_fastest_fused"] for c in cases), "cases": cases}))
 
 
 def dequant_full_model(args, torch, _capi, synth):

@@ -201,7 +201,8 @@ def test_tiled_kernel_agrees_with_the_oracle(ext, oracle):
     staged once per workgroup in LDS) forced with gemm_tiled = 2 and both tiles, on shapes small enough for the oracle:
     ragged row counts on both sides, one stage per byte group (K = 128), a tail chunk with a partial last step
     (K = 2176, 11008), several tiles of activation rows (M = 300).  Every output sums its products in the same order
-    whatever the tile, so the two tiles agree bit for bit."""
+    whatever the tile, so the two tiles agree bit for bit (with one group of waves per workgroup; with two, each on half
+    of K, the sums meet in a different order)."""
     from any_precision_amd import _capi
     for N, K in ((200, 128), (64, 1024), (130, 2176), (96, 11008), (257, 4096)):
         L = make(N, K, seed=N + K)
@@ -210,13 +211,18 @@ def test_tiled_kernel_agrees_with_the_oracle(ext, oracle):
             for M in (1, 17, 64, 65, 130, 300):
                 print(f"tiled N={N} K={K} b={b} M={M}", flush=True)
                 x, xg = _x(M, K, seed=M)
-                with _capi.tuning(gemm_tiled=2, gemm_tile=4):
+                with _capi.tuning(gemm_tiled=2, gemm_tile=4, gemm_tile_split=1):
                     small = ext.gemm_kbit(xg, q, luts[b], b)
                 with _capi.tuning(gemm_tiled=2, gemm_tile=8):
                     large = ext.gemm_kbit(xg, q, luts[b], b)
                 _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
                 assert_close_gemv(small, want, f"tiled N={N} K={K} b={b} M={M}")
                 assert torch.equal(small.view(torch.int16), large.view(torch.int16)), (N, K, b, M)
+                # two groups of waves per workgroup, each on half of K (the second idles through a last step when
+                # the number of steps is odd: K = 2176 has 5, K = 11008 has 22, K = 128 has 1 and keeps one group)
+                with _capi.tuning(gemm_tiled=2, gemm_tile=4, gemm_tile_split=2):
+                    halves = ext.gemm_kbit(xg, q, luts[b], b)
+                assert_close_gemv(halves, want, f"tiled halves N={N} K={K} b={b} M={M}")
     # one-hot activation rows return columns of the dequantised weight exactly (K = 2176: also the partial step)
     N, K = 130, 2176
     L = make(N, K, seed=N + K)
