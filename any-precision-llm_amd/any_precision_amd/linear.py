@@ -28,8 +28,9 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).
     With the tiled kernel (rows of a multiple of 128 elements, linears of at least 4096 rows): at 3 bits up to 256
     activation rows everywhere (4096 x 4096: 24-25 us against 39-43; 11008 x 4096: 48-71 against 58-73; 4096 x 11008:
-    63-65 against 78-84); at 4 bits up to 128 (11008 x 4096: 52 against 57; 4096 x 11008: 77 against 85); at 4 and 5
-    bits up to 256 on linears of fewer than 8192 rows of at most 4096 elements (4096 x 4096: 30-35 against 40-44); and
+    63-65 against 78-84); at 4 bits up to 128 (11008 x 4096: 52 against 58) and up to 256 on linears of fewer than
+    8192 rows (4096 x 4096: 26-27 against 39-45; 4096 x 11008: 65-69 against 78-84); at 5 bits up to 256 on linears of
+    fewer than 8192 rows of at most 4096 elements (4096 x 4096: 33-35 against 40-44); and
     up to 64 rows at every bit-width on linears of 8192 rows or more of at most 4096 elements (11008 x 4096, 8 bits:
     41 against 53).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising
     the weight once."""
@@ -37,7 +38,7 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
         return True
     if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
         small = out_features < 8192 and in_features <= 4096
-        if w_bits == 3 or (w_bits == 4 and rows <= 128) or (w_bits <= 5 and small):
+        if w_bits == 3 or (w_bits == 4 and (rows <= 128 or out_features < 8192)) or (w_bits == 5 and small):
             return True
         if rows <= 64 and out_features >= 8192 and in_features <= 4096:
             return True

@@ -396,7 +396,8 @@ bool gemmw_geometry(int M, int N, int K, int w_bits, GemmwGeometry *geo) {
 // matrix instruction (measured on 4096 x 4096, 11008 / 14336 x 4096, 4096 x 11008, 5120 x 5120, 8192 x 8192 at 48..512
 // rows: the larger tile wins from about 3 workgroups of the smaller one per CU on at 3 bits, from 1.3 on at 4+ bits).
 // Grids of at most one small tile per CU run it with two groups of waves, each on half of K (4096 x 4096 at 128..256
-// rows: 30 us against 37 at 4 bits, 38 against 50 at 8; 4096 x 11008: 77 against 100 at 4 bits); with more tiles than
+// rows: 38 us against 50 at 8 bits, 26 against 37 at 4 bits, where this form also has room for the pair table; 4096 x
+// 11008: 65 against 100 at 4 bits); with more tiles than
 // CUs the second group only takes LDS from the next workgroup (11008 x 4096, 256 rows, 3 bits: 71 us against 56).
 bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
     if ((K & 127) != 0 || (long long)M * K * 2 > 0xffffffffLL) return false;
@@ -419,12 +420,13 @@ bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
 
 // Where the tiled kernel is the fastest fused form (same sweep, against the K-split kernel, which serves more than 128
 // rows in chunks of 128): always beyond 128 rows; on linears of at least 8192 rows of at most 4096 elements from 64
-// rows on (11008 x 4096 at 64 rows: 26-41 us against 38-58), at 3 bits from 48; elsewhere at 3 bits from 96 rows on and
-// at 4 and 5 bits from 120 (4096 x 4096 at 128 rows: 30 / 33 us against 34 / 35; 4096 x 11008: 77 / 84 against 88 / 98).
+// rows on (11008 x 4096 at 64 rows: 26-41 us against 38-58), at 3 bits from 48; elsewhere at 3 and 4 bits from 96 rows
+// on and at 5 bits from 120 (4096 x 4096 at 128 rows: 24 / 26 / 33 us against 34 / 34 / 35; 4096 x 11008: 62 / 65 / 84
+// against 86 / 88 / 98).
 bool gemmt_pays(int M, int N, int K, int w_bits) {
     if (M > 128) return true;
     if (N >= 8192 && K <= 4096) return M >= (w_bits == 3 ? 48 : 64);
-    return w_bits == 3 ? M >= 96 : (w_bits <= 5 && M >= 120);
+    return w_bits <= 4 ? M >= 96 : (w_bits == 5 && M >= 120);
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).

@@ -34,9 +34,11 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K) {
     constexpr int NC = 1 << BITS;
-    // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 256 bytes per row).  At 4 bits that
-    // table is 1 KB per row -- too much for 64 RB rows beside the activation stages -- so 4 bits use single indices.
-    constexpr bool PAIR = BITS == 3;
+    // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 256 bytes per row): half the table reads,
+    // which are what loads the LDS port.  At 4 bits that table is 1 KB per row, 64 KB per workgroup: it pays where a CU
+    // holds one workgroup anyway (the grids that run two K halves: 4096 x 4096 at 128 rows 26 us against 31) and costs
+    // where it halves the workgroups per CU (11008 x 4096 at 256 rows: 92 us against 74), so only KH = 2 uses it.
+    constexpr bool PAIR = BITS == 3 || (BITS == 4 && KH == 2);
     constexpr int TB = PAIR ? LookupTable<BITS>::kBytes : 2 * NC;  // bytes of one row's table in LDS
     constexpr int WROWS = kGemmRows * RB;                           // weight rows per wave
     constexpr int BN = kGemmtWaves * WROWS, BM = 16 * MBW;
@@ -168,7 +170,11 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(
             static_for<NRAW>([&](auto e_c) {
                 constexpr int i = decltype(e_c)::value;
                 if constexpr (PAIR) {
-                    raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(byte_add<c>(tab_base, idx[wi][rb][i]));
+                    // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
+                    uint32_t a0;
+                    if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
+                    else a0 = tab_base + byte_offset<c, 2>(idx[wi][rb][i]);
+                    raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(a0);
                 } else {
                     uint32_t a0;
                     if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);

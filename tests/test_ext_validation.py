@@ -62,7 +62,7 @@ def test_fused_gemm_dispatch_rule():
     assert fused_gemm_pays(256, 11008, 3, 4096) and fused_gemm_pays(200, 4096, 3, 11008) and not fused_gemm_pays(257, 4096, 3, 4096)
     assert not fused_gemm_pays(100, 1024, 3, 4096) and not fused_gemm_pays(200, 4096, 3, 4000)   # narrow; rows the tiled kernel does not take
     assert fused_gemm_pays(128, 11008, 4, 4096) and not fused_gemm_pays(192, 11008, 4, 4096) and fused_gemm_pays(256, 4096, 4, 4096)
-    assert fused_gemm_pays(128, 4096, 4, 11008) and not fused_gemm_pays(129, 4096, 4, 11008)
+    assert fused_gemm_pays(128, 4096, 4, 11008) and fused_gemm_pays(256, 4096, 4, 11008) and not fused_gemm_pays(129, 8192, 4, 8192)
     assert fused_gemm_pays(256, 4096, 5, 4096) and not fused_gemm_pays(256, 4096, 6, 4096) and not fused_gemm_pays(256, 5120, 5, 5120)
     assert fused_gemm_pays(64, 14336, 8, 4096) and not fused_gemm_pays(64, 14336, 8, 4000) and not fused_gemm_pays(65, 14336, 8, 4096)
     assert fused_gemm_pays(64, 5120, 5, 13824) and not fused_gemm_pays(64, 5120, 8, 13824)      # long rows, 6 bits on
