@@ -16,7 +16,9 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_random_shapes(oracle, seed):
     import any_precision_ext as ext
+    from any_precision_amd import _capi
     rng = np.random.default_rng(seed)
+    rng2 = np.random.default_rng(seed + 100)
     for c in range(16):
         N = int(rng.choice([rng.integers(1, 70), rng.integers(70, 600), rng.integers(2040, 2100)]))
         words = int(rng.choice([rng.integers(1, 40), rng.integers(40, 400), rng.choice([128, 256, 344, 448])]))
@@ -36,3 +38,18 @@ def test_random_shapes(oracle, seed):
             assert_close_gemv(ext.gemm_kbit(xg, q, luts[b], b), want, f"gemm N={N} K={K} b={b} M={M}")
             if M <= 8:
                 assert_close_gemv(ext.matmul_kbit(xg, q, luts[b], b), want, f"matmul N={N} K={K} b={b} M={M}")
+        if K % 128 == 0:
+            # the tiled GEMM: forced with either tile and one or two K halves at the larger batch, and by the default
+            # rule beyond 128 rows (its own generator, so that the cases above stay what they were)
+            M = batches[1]
+            tile, split = int(rng2.choice([4, 8])), int(rng2.choice([1, 2]))
+            x = synth.make_x(M, K, seed=M + c)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            with _capi.tuning(gemm_tiled=2, gemm_tile=tile, gemm_tile_split=split):
+                got = ext.gemm_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
+            assert_close_gemv(got, want, f"tiled {tile}/{split} N={N} K={K} b={b} M={M}")
+            M = int(rng2.integers(129, 300))
+            print(f"random case {seed}/{c}: tiled default M={M}", flush=True)
+            x = synth.make_x(M, K, seed=M + c)
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(ext.gemm_kbit(torch.from_numpy(x).cuda(), q, luts[b], b), want, f"tiled N={N} K={K} b={b} M={M}")
