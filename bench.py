@@ -137,7 +137,7 @@ def main():
         need = int(args.pool_gb * 1e9 / (3 * N * K / 8)) + 1
         sets = max(need, len(idxs) * args.pool)
         pools[(N, K)] = WeightPool(torch, N, K, sets, gen)
-    batches = (1, 2, 4, 8, 16, 32)
+    batches = (1, 2, 4, 8, 16, 32, 128, 256)
     xb = {(M, K): torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
           for K in {K for _, _, K in shapes} for M in batches}
     for P in pools.values():
@@ -331,13 +331,26 @@ def main():
                                       "write_only_us": round(us_write, 2), "read_only_us": us_read,
                                       "frac_of_write_floor": round(us_write / us, 4)})
             del outs
-        # batches: matmul_kbit for M <= 8 (MFMA kernel from 5 rows on), fused gemm_kbit for 16 and 32 rows
+        # batches: matmul_kbit for M <= 8 (MFMA kernel from 5 rows on), fused gemm_kbit beyond (K-split kernel at 16 and
+        # 32 rows, tiled kernel at 128 and 256), there beside dequant_kbit + library GEMM on the same weight sets
+        import any_precision_ext as ext
         for (N, K) in pools:
             for b in (3, 4, 8):
                 row = {"N": N, "K": K, "w_bits": b}
                 for M in batches:
                     fn = lib.ap_matmul_kbit if M <= 8 else lib.ap_gemm_kbit
-                    row[f"us_M{M}"] = round(time_graph(lambda st: launch(N, K, b, st, M, fn), 24), 2)
+                    row[f"us_M{M}"] = round(time_graph(lambda st: launch(N, K, b, st, M, fn), 24 if M <= 32 else 8), 2)
+                    if M >= 128:
+                        P = pools[(N, K)]
+
+                        def pair(st):
+                            j = cursor[(N, K)] = (cursor[(N, K)] + 1) % P.sets
+                            torch.matmul(xb[(M, K)], ext.dequant_kbit(P.qweight[j], P.luts[b][j], b).T, out=P.out[:M])
+
+                        with torch.cuda.stream(side):   # the library GEMM sets itself up on first use: not inside a capture
+                            pair(side.cuda_stream)
+                            side.synchronize()
+                        row[f"dequant_matmul_us_M{M}"] = round(time_graph(pair, 8), 2)
                 batch_table.append(row)
 
     # ---- compact figures for the other configurations (each has a --workload of its own with the full
@@ -487,7 +500,7 @@ def main():
                 for r in dequant_table:
                     f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | {r['us']:.1f} | {r['GBps']:.0f} | {100 * r['frac']:.1f} |\n")
             if batch_table:
-                f.write("\nus per launch by batch (M <= 8: matmul_kbit; 16, 32: gemm_kbit)\n\n")
+                f.write("\nus per launch by batch (M <= 8: matmul_kbit; 16 and more: gemm_kbit)\n\n")
                 f.write("| N x K | w_bits | " + " | ".join(f"M={M}" for M in batches) + " |\n|---|---|" + "---|" * len(batches) + "\n")
                 for r in batch_table:
                     f.write(f"| {r['N']}x{r['K']} | {r['w_bits']} | " + " | ".join(f"{r[f'us_M{M}']:.1f}" for M in batches) + " |\n")
