@@ -26,21 +26,28 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     than 4096 elements, from 6 bits on linears of 5120 rows or more (5120 x 13824, 8 bits: 121 us against 86)
     and from 5 bits on linears of at most 2048 rows (1024 x 8192); up to 128 on linears of 4096..8191
     rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).
-    With the tiled kernel (rows of a multiple of 128 elements, linears of at least 4096 rows): at 3 bits up to 256
-    activation rows everywhere (4096 x 4096: 24-25 us against 39-43; 11008 x 4096: 48-71 against 58-73; 4096 x 11008:
-    63-65 against 78-84); at 4 bits up to 128 (11008 x 4096: 52 against 58) and up to 256 on linears of fewer than
-    8192 rows (4096 x 4096: 26-27 against 39-45; 4096 x 11008: 65-69 against 78-84); at 5 bits up to 256 on linears of
-    fewer than 8192 rows of at most 4096 elements (4096 x 4096: 33-35 against 40-44); and
-    up to 64 rows at every bit-width on linears of 8192 rows or more of at most 4096 elements (11008 x 4096, 8 bits:
-    41 against 53).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising
-    the weight once."""
+    With the tiled kernel (rows of a multiple of 128 elements, linears of at least 4096 rows; measured on the linear
+    shapes of the 7B / 8B / 13B / 70B layers at 48..256 activation rows) the fused form wins up to 256 rows:
+    at 3 bits everywhere (4096 x 4096: 24-25 us against 39-43; 11008 x 4096: 41-57 against 58-73; 28672 x 8192 at 128
+    rows: 118 against 201); at 4 bits up to 128 rows everywhere and up to 256 on linears of 4096 rows or of fewer than
+    8192 rows of at most 5120 elements (4096 x 4096: 26-27 against 39-45); at 5 and 6 bits up to 128 rows on linears of
+    8192 rows or more (13824 x 5120: 71-73 against 74-80; 28672 x 8192: 153-160 against 214-223) and on those small
+    ones (5120 x 5120: 40-42 against 52), at 5 bits up to 256 on 4096 x 4096; at 7 and 8 bits up to 64 rows on wide
+    linears (11008 x 4096: 41 against 53; 28672 x 8192: 139 against 232) and up to 128 on the small ones (5120 x 5120:
+    48 against 52).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising the
+    weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
     if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
-        small = out_features < 8192 and in_features <= 4096
-        if w_bits == 3 or (w_bits == 4 and (rows <= 128 or out_features < 8192)) or (w_bits == 5 and small):
+        small = out_features < 8192 and in_features <= 5120
+        wide = out_features > 10240 or (out_features >= 8192 and in_features <= 4096)
+        if w_bits == 3:
             return True
-        if rows <= 64 and out_features >= 8192 and in_features <= 4096:
+        if w_bits == 4 and (rows <= 128 or out_features <= 4096 or small):
+            return True
+        if w_bits in (5, 6) and ((rows <= 128 and (out_features >= 8192 or small)) or (w_bits == 5 and small and in_features <= 4096)):
+            return True
+        if w_bits >= 7 and ((rows <= 64 and wide) or (rows <= 128 and small)):
             return True
     if rows <= min(64, GEMM_MAX_M):
         if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):

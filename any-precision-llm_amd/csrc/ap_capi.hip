@@ -418,15 +418,20 @@ bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
     return geo->grid_m <= 65535;
 }
 
-// Where the tiled kernel is the fastest fused form (same sweep, against the K-split kernel, which serves more than 128
-// rows in chunks of 128): always beyond 128 rows; on linears of at least 8192 rows of at most 4096 elements from 64
-// rows on (11008 x 4096 at 64 rows: 26-41 us against 38-58), at 3 bits from 48; elsewhere at 3 and 4 bits from 96 rows
-// on and at 5 bits from 120 (4096 x 4096 at 128 rows: 24 / 26 / 33 us against 34 / 34 / 35; 4096 x 11008: 62 / 65 / 84
-// against 86 / 88 / 98).
+// Where the tiled kernel is the fastest fused form (same sweep, and the linear shapes of the 7B / 8B / 13B / 70B layers
+// at 48..256 rows, against the K-split kernel, which serves more than 128 rows in chunks of 128): from 120 rows on
+// everywhere (4096 x 4096 at 128 rows: 24 / 26 / 33 / 37 us at 3 / 4 / 5 / 8 bits against 34-36; rows of more than 4096
+// elements at 8 bits: 1.8-2x, e.g. 13824 x 5120 83 us against 171).  Its time does not depend on the number of
+// activation rows within a tile of 64, the K-split kernel's grows with them, so wide linears -- at least 8192 rows of at
+// most 4096 elements, or more than 10240 rows of any length -- cross over at 40..48 rows (11008 x 4096 at 64 rows:
+// 26-41 us against 38-58; 13824 x 5120: 33-53 against 63-100; 28672 x 8192 at 48 rows: 81 against 124).  Linears of
+// 5120..10240 rows of more than 4096 elements from 96 rows on at every bit-width (5120 x 5120 at 5 bits: 40 us against
+// 63); the rest (4096 rows) from 96 rows on at 3 and 4 bits.
 bool gemmt_pays(int M, int N, int K, int w_bits) {
-    if (M > 128) return true;
-    if (N >= 8192 && K <= 4096) return M >= (w_bits == 3 ? 48 : 64);
-    return w_bits <= 4 ? M >= 96 : (w_bits == 5 && M >= 120);
+    if (M >= 120) return true;
+    if ((N >= 8192 && K <= 4096) || N > 10240) return M >= (w_bits <= 4 ? 40 : 48);
+    if (N >= 5120 && K > 4096) return M >= 96;
+    return w_bits <= 4 && M >= 96;
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).

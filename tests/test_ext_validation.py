@@ -54,16 +54,18 @@ def test_fused_gemm_dispatch_rule():
     AnyPrecisionLinear.py:60-62)."""
     from any_precision_amd.linear import fused_gemm_pays
     assert all(fused_gemm_pays(m, n, b) for m in (9, 32) for n in (4096, 14336) for b in (3, 8))
-    assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6) and not fused_gemm_pays(64, 14336, 6, 8192)
+    assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6) and fused_gemm_pays(64, 14336, 6, 8192)
     assert not fused_gemm_pays(65, 4096, 5) and not fused_gemm_pays(65, 4096, 5, 11008) and not fused_gemm_pays(129, 4096, 6, 4096)
-    assert fused_gemm_pays(128, 4096, 8, 4096) and not fused_gemm_pays(128, 11008, 5, 4096)
+    assert fused_gemm_pays(128, 4096, 8, 4096) and fused_gemm_pays(128, 11008, 5, 4096) and not fused_gemm_pays(128, 11008, 8, 4096)
     # the tiled kernel: 3 bits to 256 rows on linears of 4096 rows or more, 4 bits to 128, 4-5 bits to 256 on small linears,
-    # every bit-width to 64 rows on wide linears of short rows
+    # 5-6 bits to 128 on linears of 8192 rows or more, every bit-width to 64 rows on wide linears
     assert fused_gemm_pays(256, 11008, 3, 4096) and fused_gemm_pays(200, 4096, 3, 11008) and not fused_gemm_pays(257, 4096, 3, 4096)
     assert not fused_gemm_pays(100, 1024, 3, 4096) and not fused_gemm_pays(200, 4096, 3, 4000)   # narrow; rows the tiled kernel does not take
     assert fused_gemm_pays(128, 11008, 4, 4096) and not fused_gemm_pays(192, 11008, 4, 4096) and fused_gemm_pays(256, 4096, 4, 4096)
     assert fused_gemm_pays(128, 4096, 4, 11008) and fused_gemm_pays(256, 4096, 4, 11008) and not fused_gemm_pays(129, 8192, 4, 8192)
     assert fused_gemm_pays(256, 4096, 5, 4096) and not fused_gemm_pays(256, 4096, 6, 4096) and not fused_gemm_pays(256, 5120, 5, 5120)
     assert fused_gemm_pays(64, 14336, 8, 4096) and not fused_gemm_pays(64, 14336, 8, 4000) and not fused_gemm_pays(65, 14336, 8, 4096)
+    assert fused_gemm_pays(128, 28672, 6, 8192) and not fused_gemm_pays(129, 28672, 6, 8192) and fused_gemm_pays(64, 28672, 8, 8192)
+    assert not fused_gemm_pays(64, 8192, 8, 8192) and fused_gemm_pays(128, 5120, 8, 5120) and not fused_gemm_pays(128, 5120, 6, 13824)
     assert fused_gemm_pays(64, 5120, 5, 13824) and not fused_gemm_pays(64, 5120, 8, 13824)      # long rows, 6 bits on
     assert fused_gemm_pays(64, 1024, 8, 4096) and not fused_gemm_pays(64, 1024, 5, 8192)        # narrow, long rows
