@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libanyprec_hip.so")
 
 AP_OK = 0
 AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT, AP_EKNOB = -1, -2, -3, -4, -5, -6, -7
-AP_ABI_VERSION = 6
+AP_ABI_VERSION = 7
 
 if not os.path.exists(LIB_PATH):
     raise ModuleNotFoundError(
@@ -37,6 +37,9 @@ _pi = ctypes.POINTER(ctypes.c_int)
 _pvp = ctypes.POINTER(ctypes.c_void_p)
 lib.ap_matmul_kbit_group.argtypes = [_vp, _ci, _pvp, _pvp, _pvp, _pi, _ci, _ci, _ci, _vp]
 lib.ap_matmul_kbit_group.restype = _ci
+_pll = ctypes.POINTER(ctypes.c_longlong)
+lib.ap_gemm_kbit_group.argtypes = [_vp, _ci, _pvp, _pvp, _pvp, _pi, _pll, _ci, _ci, _ci, _vp]
+lib.ap_gemm_kbit_group.restype = _ci
 lib.ap_matmul_kbit_geometry.argtypes = [_ci, _ci, _ci, _ci, _pi, _pi, _pi, _pi]
 lib.ap_matmul_kbit_geometry.restype = _ci
 lib.ap_probe_stream.argtypes = [_vp, ctypes.c_longlong, _vp, ctypes.c_longlong, _vp, _ci, _vp]
@@ -71,7 +74,7 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
            "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_probe_write", "ap_matmul_kbit_route", "ap_matmul_kbit_group_route",
-           "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu", "ap_decode_advance")
+           "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu", "ap_decode_advance", "ap_gemm_kbit_group")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
 
@@ -82,6 +85,15 @@ def matmul_group(x_ptr: int, qweights, luts, outs, rows, M: int, K: int, w_bits:
     arr = ctypes.c_void_p * n
     return lib.ap_matmul_kbit_group(x_ptr, n, arr(*qweights), arr(*luts), arr(*outs), (ctypes.c_int * n)(*rows),
                                     M, K, w_bits, stream)
+
+
+def gemm_group(x_ptr: int, qweights, luts, outs, rows, ldo, M: int, K: int, w_bits: int, stream: int) -> int:
+    """ap_gemm_kbit_group on raw device addresses (lists of equal length <= GROUP_MAX; ldo: row strides or None)."""
+    n = len(qweights)
+    arr = ctypes.c_void_p * n
+    strides = None if ldo is None else (ctypes.c_longlong * n)(*ldo)
+    return lib.ap_gemm_kbit_group(x_ptr, n, arr(*qweights), arr(*luts), arr(*outs), (ctypes.c_int * n)(*rows), strides,
+                                  M, K, w_bits, stream)
 
 
 def strerror(code: int) -> str:

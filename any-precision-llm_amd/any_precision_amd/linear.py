@@ -14,9 +14,10 @@ import torch
 import torch.nn as nn
 
 try:
-    from any_precision_ext import matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, GEMM_MAX_M
+    from any_precision_ext import (matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, gemm_kbit_group,
+                                   GEMM_MAX_M)
 except ModuleNotFoundError:
-    matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, GEMM_MAX_M = None, None, None, None, None, 0
+    matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, gemm_kbit_group, GEMM_MAX_M = (None,) * 6 + (0,)
 
 
 def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int = 0) -> bool:
@@ -56,23 +57,42 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     return rows <= min(128, GEMM_MAX_M) and 4096 <= out_features < 8192 and 0 < in_features <= 4096
 
 
+def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bool:
+    """Whether ONE launch of the tiled GEMM over linears that share their input (``gemm_kbit_group``) beats calling them
+    one by one, each through whatever ``fused_gemm_pays`` picks (measured on the q/k/v and gate/up sets of the
+    Llama-2-7B / Llama-3-8B / 13B layers at 48..256 rows): from 33 rows on (below, the K-split kernel module by
+    module) up to 256 rows at up to 6 bits (q/k/v of the 7B layer at 128 rows, 3 bits: 39 us against 69 one by one and
+    129 for three dequant + GEMM pairs; gate/up at 256 rows, 5 bits: 125 against 146); at 7 and 8 bits up to 64 rows,
+    and up to 128 where every member has fewer than 8192 rows (q/k/v at 8 bits: 66 against 127; gate/up: 129 against
+    114 for the pairs)."""
+    if in_features % 128 or not 32 < rows <= 256 or sum(out_features) < 4096:
+        return False
+    return w_bits <= 6 or rows <= 64 or (rows <= 128 and max(out_features) < 8192)
+
+
 def forward_group(modules, x, precision=None, concat=False):
     """``[m(x, precision=precision) for m in modules]`` for linears that share their input (the
     q/k/v or gate/up projections of a decoder layer); with ``concat`` the results joined along
     the last dimension.  Up to 8 activation rows and 4 modules they go through ``matmul_kbit_group``, which
     issues ONE launch wherever the dot-product kernel serves the set (always up to 4 rows; at 5..8 rows for
-    sets with narrow members and some 5-8-bit cases) and a launch per member otherwise; beyond, module by module.  The reference has no counterpart (its ``fuse_layers`` is a
-    stub, AnyPrecisionForCausalLM.py:168-172)."""
+    sets with narrow members and some 5-8-bit cases) and a launch per member otherwise; beyond 32 rows through
+    ``gemm_kbit_group`` (one launch of the tiled GEMM) where the fused form pays for the set; else module by module.
+    The reference has no counterpart (its ``fuse_layers`` is a stub, AnyPrecisionForCausalLM.py:168-172)."""
     rows = x.numel() // x.shape[-1]
     w_bits = modules[0].precision if precision is None else precision
     x = x.contiguous()
-    if rows > 8 or not 2 <= len(modules) <= 4 or any(
-            m.in_features != modules[0].in_features for m in modules):
+    K = modules[0].in_features
+    same_input = 2 <= len(modules) <= 4 and all(m.in_features == K for m in modules)
+    # beyond 32 rows: one launch of the tiled GEMM (three 4096 x 4096 projections at 128 rows fill the chip that one of
+    # them leaves half idle); up to 32 rows the K-split kernel, module by module, is faster
+    tiled_set = same_input and fused_set_pays(rows, [m.out_features for m in modules], w_bits, K)
+    if not same_input or (rows > 8 and not tiled_set):
         outs = [m(x, precision=w_bits) for m in modules]
         return torch.cat(outs, dim=-1) if concat else outs
     has_bias = any(m.bias is not None for m in modules)
-    res = matmul_kbit_group(x, [m.qweight for m in modules], [m._buffers[f"lut{w_bits}"] for m in modules], w_bits,
-                            concat=concat and not has_bias)
+    group_op = gemm_kbit_group if rows > 8 else matmul_kbit_group
+    res = group_op(x, [m.qweight for m in modules], [m._buffers[f"lut{w_bits}"] for m in modules], w_bits,
+                   concat=concat and not has_bias)
     if not has_bias:
         return res
     for m, o in zip(modules, res):

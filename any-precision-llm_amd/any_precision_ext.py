@@ -22,7 +22,7 @@ import torch
 
 from any_precision_amd import _capi
 
-__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "matmul_kbit_group", "matmul_kbit_swiglu", "GEMM_MAX_M"]
+__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "gemm_kbit_group", "matmul_kbit_group", "matmul_kbit_swiglu", "GEMM_MAX_M"]
 
 GEMM_MAX_M = _capi.GEMM_MAX_M
 
@@ -120,6 +120,46 @@ def matmul_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int, concat: bo
                                 [o.data_ptr() for o in outs], [N for N, _ in shapes], M, K, w_bits,
                                 torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "matmul_kbit_group")
+    if concat:
+        return joint if joint is not None else torch.cat(outs, dim=-1)
+    return outs
+
+
+def gemm_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int, concat: bool = False):
+    """``[gemm_kbit(in_, q, t, w_bits) for q, t in zip(qweights, luts)]`` for up to GROUP_MAX linears that share the
+    input and the bit-width, any number of activation rows: ONE launch of the tiled kernel where it serves the set
+    (rows of a multiple of 128 elements) and pays, a launch per member otherwise.  ``concat=True`` returns the results
+    joined along the last dimension as one tensor (written side by side into one allocation where the tiled kernel
+    serves the set; joined with ``torch.cat`` otherwise).  No counterpart in the reference."""
+    if len(qweights) != len(luts) or not 1 <= len(qweights) <= _capi.GROUP_MAX:
+        raise ValueError(f"gemm_kbit_group: need 1..{_capi.GROUP_MAX} (qweight, lut) pairs")
+    shapes = [_check_weight(q, t, w_bits, "gemm_kbit_group") for q, t in zip(qweights, luts)]
+    K = shapes[0][1]
+    if any(k != K for _, k in shapes):
+        raise ValueError("gemm_kbit_group: all members must have the same in_features")
+    if in_.dtype != torch.float16:
+        raise ValueError(f"gemm_kbit_group: input must be float16, got {in_.dtype}")
+    if any(q.device != in_.device for q in qweights):
+        raise ValueError("gemm_kbit_group: input and weights must be on one device")
+    if in_.dim() < 1 or in_.shape[-1] != K:
+        raise ValueError(f"gemm_kbit_group: input last dim must be K={K}, got {tuple(in_.shape)}")
+    M = in_.numel() // K if K else 0
+    if M < 1:
+        raise ValueError("gemm_kbit_group: empty input")
+    if not in_.is_contiguous():
+        raise ValueError("gemm_kbit_group: input must be contiguous")
+    rows = [N for N, _ in shapes]
+    with torch.cuda.device(in_.device):
+        joint, ldo = None, None
+        if concat and K % 128 == 0:      # the tiled kernel writes rows that are not dense
+            joint = torch.empty(in_.shape[:-1] + (sum(rows),), dtype=torch.float16, device=in_.device)
+            outs = list(torch.split(joint, rows, dim=-1))
+            ldo = [sum(rows)] * len(rows)
+        else:
+            outs = [torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device) for N in rows]
+        rc = _capi.gemm_group(in_.data_ptr(), [q.data_ptr() for q in qweights], [t.data_ptr() for t in luts],
+                              [o.data_ptr() for o in outs], rows, ldo, M, K, w_bits, torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "gemm_kbit_group")
     if concat:
         return joint if joint is not None else torch.cat(outs, dim=-1)
     return outs

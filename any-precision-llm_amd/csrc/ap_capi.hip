@@ -399,10 +399,10 @@ bool gemmw_geometry(int M, int N, int K, int w_bits, GemmwGeometry *geo) {
 // rows: 38 us against 50 at 8 bits, 26 against 37 at 4 bits, where this form also has room for the pair table; 4096 x
 // 11008: 65 against 100 at 4 bits); with more tiles than
 // CUs the second group only takes LDS from the next workgroup (11008 x 4096, 256 rows, 3 bits: 71 us against 56).
-bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
-    if ((K & 127) != 0 || (long long)M * K * 2 > 0xffffffffLL) return false;
+bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *geo) {
+    if ((K & 127) != 0 || (long long)M * K * 2 > 0xffffffffLL || tiles_n > 0x7fffffffLL) return false;
     const int forced = knob(kGemmTile), force_kh = knob(kGemmTileSplit);
-    const long long small = (long long)((N + 63) / 64) * ((M + 63) / 64);  // tiles of 64 x 64
+    const long long small = tiles_n * ((M + 63) / 64);  // tiles of 64 x 64
     int mbw = 4;
     if (forced > 0) {
         if (forced != 4 && forced != 8) return false;
@@ -413,7 +413,7 @@ bool gemmt_geometry(int M, int N, int K, int w_bits, GemmtGeometry *geo) {
     geo->mbw = mbw;
     // two K halves need at least two steps of 512 elements
     geo->kh = mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && small <= cu_count())) ? 2 : 1;
-    geo->grid_n = (N + 63) / 64;
+    geo->grid_n = (int)tiles_n;  // tiles of 64 weight rows (of all linears of the launch)
     geo->grid_m = (M + 16 * mbw - 1) / (16 * mbw);
     return geo->grid_m <= 65535;
 }
@@ -847,6 +847,30 @@ int ap_matmul_kbit_swiglu(const uint16_t *x, const uint32_t *qweight_gate, const
     return launch_status();
 }
 
+// One launch of the tiled kernel over `count` linears (arguments already checked; geo from gemmt_geometry over all tiles).
+int run_gemmt(const GemmtGeometry &geo, const uint16_t *x, int count, const uint32_t *const *qweight, const uint16_t *const *lut,
+              uint16_t *const *out, const int *N, const long long *ldo, int M, int K, int w_bits, hipStream_t st) {
+    GemmtMembers mem = {};
+    mem.count = count;
+    for (int g = 0; g < count; g++) {
+        mem.qweight[g] = qweight[g];
+        mem.lut[g] = lut[g];
+        mem.out[g] = out[g];
+        mem.N[g] = N[g];
+        mem.ldo[g] = ldo ? ldo[g] : N[g];
+        mem.tile0[g + 1] = mem.tile0[g] + (N[g] + 63) / 64;
+    }
+    switch (w_bits) {
+        case 3: launch_gemmt<3>(geo, x, mem, M, K, st); break;
+        case 4: launch_gemmt<4>(geo, x, mem, M, K, st); break;
+        case 5: launch_gemmt<5>(geo, x, mem, M, K, st); break;
+        case 6: launch_gemmt<6>(geo, x, mem, M, K, st); break;
+        case 7: launch_gemmt<7>(geo, x, mem, M, K, st); break;
+        default: launch_gemmt<8>(geo, x, mem, M, K, st); break;
+    }
+    return launch_status();
+}
+
 int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
                  int w_bits, void *stream) {
     if (!x || !qweight || !lut || !out) return AP_ENULL;
@@ -858,18 +882,8 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
     {
         GemmtGeometry tgeo;
         const int mode = knob(kGemmTiled);
-        if (mode > 0 && gemmt_geometry(M, N, K, w_bits, &tgeo) && (mode >= 2 || gemmt_pays(M, N, K, w_bits))) {
-            hipStream_t st = static_cast<hipStream_t>(stream);
-            switch (w_bits) {
-                case 3: launch_gemmt<3>(tgeo, x, qweight, lut, out, M, N, K, st); break;
-                case 4: launch_gemmt<4>(tgeo, x, qweight, lut, out, M, N, K, st); break;
-                case 5: launch_gemmt<5>(tgeo, x, qweight, lut, out, M, N, K, st); break;
-                case 6: launch_gemmt<6>(tgeo, x, qweight, lut, out, M, N, K, st); break;
-                case 7: launch_gemmt<7>(tgeo, x, qweight, lut, out, M, N, K, st); break;
-                default: launch_gemmt<8>(tgeo, x, qweight, lut, out, M, N, K, st); break;
-            }
-            return launch_status();
-        }
+        if (mode > 0 && gemmt_geometry(M, (N + 63) / 64, K, w_bits, &tgeo) && (mode >= 2 || gemmt_pays(M, N, K, w_bits)))
+            return run_gemmt(tgeo, x, 1, &qweight, &lut, &out, &N, nullptr, M, K, w_bits, static_cast<hipStream_t>(stream));
     }
     // one launch serves up to kGemmMaxM activation rows; more go in chunks of that many, in order (the planes
     // are re-read per chunk; row offsets of 128 rows keep x and out 16-byte aligned for every K and N that passed)
@@ -877,6 +891,44 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
         const int rows = M - m0 < kGemmMaxM ? M - m0 : kGemmMaxM;
         const int r = run_gemm(x + (size_t)m0 * K, qweight, lut, out + (size_t)m0 * N, rows, N, K, w_bits,
                                static_cast<hipStream_t>(stream));
+        if (r != AP_OK) return r;
+    }
+    return AP_OK;
+}
+
+int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight, const uint16_t *const *lut,
+                       uint16_t *const *out, const int *N, const long long *ldo, int M, int K, int w_bits, void *stream) {
+    if (!x || !qweight || !lut || !out || !N) return AP_ENULL;
+    if (count < 1 || count > kGemmtMaxGroup) return AP_ELIMIT;
+    if (M < 1) return AP_EBATCH;
+    long long tiles = 0, rows = 0;
+    bool strided = false;
+    for (int g = 0; g < count; g++) {
+        if (!qweight[g] || !lut[g] || !out[g]) return AP_ENULL;
+        const int rc = check_common(N[g], K, w_bits);
+        if (rc != AP_OK) return rc;
+        if (!aligned16(qweight[g]) || !aligned16(lut[g])) return AP_EALIGN;
+        if (ldo && ldo[g] < N[g]) return AP_ESHAPE;
+        strided = strided || (ldo && ldo[g] != N[g]);
+        tiles += (N[g] + 63) / 64;
+        rows += N[g];
+    }
+    if (!aligned16(x)) return AP_EALIGN;
+    drain_stale_error();
+    GemmtGeometry tgeo;
+    const int mode = knob(kGemmTiled);
+    const bool fits = gemmt_geometry(M, tiles, K, w_bits, &tgeo);
+    // Tiles of different members run side by side, and the launch costs about what its largest member alone would,
+    // while the K-split kernel's launches add up: measured on the q/k/v and gate/up sets of the 7B / 8B / 13B layers at
+    // 48..256 rows the one launch is 1.1-3x faster than the members one by one (q/k/v of the 7B layer at 128 rows,
+    // 3 bits: 39 us against 69; of the 13B layer at 64 rows: 31 against 94) wherever there are more than 32 rows.
+    const bool pays = M > 32;
+    (void)rows;
+    if (fits && (strided || (count > 1 && mode > 0 && (mode >= 2 || pays))))
+        return run_gemmt(tgeo, x, count, qweight, lut, out, N, ldo, M, K, w_bits, static_cast<hipStream_t>(stream));
+    if (strided) return AP_ESHAPE;  // only the tiled kernel writes rows that are not dense
+    for (int g = 0; g < count; g++) {
+        const int r = ap_gemm_kbit(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, stream);
         if (r != AP_OK) return r;
     }
     return AP_OK;

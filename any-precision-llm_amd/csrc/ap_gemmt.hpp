@@ -14,6 +14,8 @@
 //     that the 16 rows of an operand read hit 16 different bank groups;
 //   * accumulators (RB x MBW tiles of 16 x 16) stay in registers over the whole K loop: no K-split, no combine.
 // Per stage a wave issues 4 x RB x MBW matrix instructions between two barriers.  K must be a multiple of 128.
+// One launch serves up to four linears that share x (q/k/v, gate/up): their tiles of 64 weight rows are numbered through
+// (GemmtMembers), which fills the chip where one linear alone leaves CUs idle.
 #pragma once
 #include <type_traits>
 
@@ -30,9 +32,8 @@ namespace ap {
 // order).  Twice the waves per tile: for grids that leave CUs with one workgroup of four waves, where no pipe is busy
 // and waves wait for each other's LDS round trips.
 template <int BITS, int RB, int MBW, int KH>
-__global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(
-    const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
-    half_t *__restrict__ out, int M, int N, int K) {
+__global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(const half_t *__restrict__ x, const GemmtMembers mem,
+                                                                             int M, int K) {
     constexpr int NC = 1 << BITS;
     // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 256 bytes per row): half the table reads,
     // which are what loads the LDS port.  At 4 bits that table is 1 KB per row, 64 KB per workgroup: it pays where a CU
@@ -54,8 +55,18 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(
     const int tid = wv * kWave + lane;                            // thread within the half
     const int col = lane & 15, grp = lane >> 4;
     const int W = K >> 5;
+    // the linear this tile belongs to (workgroup-uniform) and the tile's place in it
+    int g = 0;
+#pragma unroll
+    for (int i = 1; i < kGemmtMaxGroup; i++)
+        if (i < mem.count && (int)blockIdx.x >= mem.tile0[i]) g = i;
+    const uint32_t *__restrict__ qweight = mem.qweight[g];
+    const half_t *__restrict__ lut = reinterpret_cast<const half_t *>(mem.lut[g]);
+    half_t *__restrict__ out = reinterpret_cast<half_t *>(mem.out[g]);
+    const int N = mem.N[g];
+    const long long ldo = mem.ldo[g];
+    const int nb = ((int)blockIdx.x - mem.tile0[g]) * BN;  // first weight row of the workgroup
     const size_t plane_stride = (size_t)N * W;
-    const int nb = blockIdx.x * BN;     // first weight row of the workgroup
     const int n0 = nb + wv * WROWS;     // ... of this wave
     const int m0 = blockIdx.y * BM;     // first activation row of the tile
     const int steps = (W + 15) >> 4;    // 16 words of every row per step
@@ -289,7 +300,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const int m = m0 + mb * 16 + 4 * grp + v;
-                if (m < M && n < N) out[(size_t)m * N + n] = (half_t)acc[rb][mb][v];
+                if (m < M && n < N) out[(size_t)m * ldo + n] = (half_t)acc[rb][mb][v];
             }
     }
 }

@@ -9,22 +9,19 @@
 namespace ap {
 
 template <int BITS>
-void launch_gemmt(const GemmtGeometry &geo, const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
-                  uint16_t *out, int M, int N, int K, hipStream_t stream) {
-    const half_t *xh = reinterpret_cast<const half_t *>(x), *lh = reinterpret_cast<const half_t *>(lut);
-    half_t *oh = reinterpret_cast<half_t *>(out);
+void launch_gemmt(const GemmtGeometry &geo, const uint16_t *x, const GemmtMembers &members, int M, int K, hipStream_t stream) {
+    const half_t *xh = reinterpret_cast<const half_t *>(x);
     const dim3 block(kWave, kGemmtWaves * geo.kh), grid(geo.grid_n, geo.grid_m);
     // one block of 16 weight rows per wave: two measured slower on every shape (a quarter of the workgroups, and the
     // LDS traffic per matrix instruction falls by less than a third)
     if (geo.mbw == 8)
-        gemmt_kbit_kernel<BITS, 1, 8, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+        gemmt_kbit_kernel<BITS, 1, 8, 1><<<grid, block, 0, stream>>>(xh, members, M, K);
     else if (geo.kh == 2)
-        gemmt_kbit_kernel<BITS, 1, 4, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+        gemmt_kbit_kernel<BITS, 1, 4, 2><<<grid, block, 0, stream>>>(xh, members, M, K);
     else
-        gemmt_kbit_kernel<BITS, 1, 4, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+        gemmt_kbit_kernel<BITS, 1, 4, 1><<<grid, block, 0, stream>>>(xh, members, M, K);
 }
 
-template void launch_gemmt<AP_BITS>(const GemmtGeometry &, const uint16_t *, const uint32_t *, const uint16_t *, uint16_t *,
-                                    int, int, int, hipStream_t);
+template void launch_gemmt<AP_BITS>(const GemmtGeometry &, const uint16_t *, const GemmtMembers &, int, int, hipStream_t);
 
 }  // namespace ap

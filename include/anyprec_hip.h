@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 6
+#define AP_ABI_VERSION 7
 
 enum {
     AP_OK = 0,
@@ -98,6 +98,20 @@ int ap_matmul_kbit_swiglu(const uint16_t *x, const uint32_t *qweight_gate, const
  * fp32 accumulation, fp16 result. */
 int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut,
                  uint16_t *out, int M, int N, int K, int w_bits, void *stream);
+
+/* ap_gemm_kbit for 1..4 linears that share x, K and w_bits (the q/k/v or gate/up projections of a decoder
+ * layer on a batch of rows): out[g][M, N[g]] = x[M,K] . dequant(qweight[g], lut[g])^T.  Where the tiled
+ * kernel serves the set (K % 128 == 0) and pays for it taken as one linear of all its rows, ONE launch
+ * whose tiles of 64 weight rows run through the members -- three 4096 x 4096 projections at 128 rows fill
+ * the chip that one of them leaves half idle; otherwise one ap_gemm_kbit per member, in order.
+ * ldo (may be NULL: dense results) gives the distance in elements between consecutive rows of each
+ * out[g], so that the results can be written side by side into one [M, sum N] array (out[g] = its
+ * column offset, ldo[g] = sum N); results that are not dense need the tiled kernel: AP_ESHAPE if
+ * K % 128 != 0 then.  No counterpart in the reference (its fuse_layers hook is a stub,
+ * AnyPrecisionForCausalLM.py:168-172).  AP_ELIMIT for count outside 1..4. */
+int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight,
+                       const uint16_t *const *lut, uint16_t *const *out, const int *N,
+                       const long long *ldo, int M, int K, int w_bits, void *stream);
 
 /* Human-readable text for a return code of the functions above. */
 const char *ap_strerror(int code);

@@ -95,6 +95,21 @@ def test_decode_step_argument_errors_need_no_gpu():
     assert att(kc=fake + 8) == _capi.AP_EALIGN
 
 
+def test_gemm_group_argument_errors_need_no_gpu():
+    from any_precision_amd import _capi
+    fake = 4096
+    call = lambda **kw: _capi.gemm_group(kw.get("x", fake), kw.get("q", [fake, fake]), kw.get("t", [fake, fake]),
+                                         kw.get("o", [fake, fake]), kw.get("N", [64, 64]), kw.get("ldo"), kw.get("M", 40),
+                                         kw.get("K", 128), kw.get("b", 3), 0)
+    assert call(x=None) == _capi.AP_ENULL and call(q=[fake, None]) == _capi.AP_ENULL
+    assert call(q=[fake] * 5, t=[fake] * 5, o=[fake] * 5, N=[64] * 5) == _capi.AP_ELIMIT
+    assert call(M=0) == _capi.AP_EBATCH
+    assert call(b=2) == _capi.AP_EBITS
+    assert call(K=100) == _capi.AP_ESHAPE and call(N=[64, 0]) == _capi.AP_ESHAPE
+    assert call(ldo=[128, 63]) == _capi.AP_ESHAPE          # rows of a result overlap
+    assert call(t=[fake, fake + 2]) == _capi.AP_EALIGN and call(x=fake + 8) == _capi.AP_EALIGN
+
+
 def test_geometry_covers_rows_and_words():
     from any_precision_amd import _capi
     for M in (1, 2, 4, 8):

@@ -271,3 +271,47 @@ def test_tiled_kernel_by_default_beyond_128_rows(ext, oracle):
             g.replay()
             torch.cuda.synchronize()
             assert torch.equal(out.view(torch.int16), got.view(torch.int16)), rep
+
+
+def test_group_of_linears_in_one_tiled_launch(ext, oracle):
+    """gemm_kbit_group: linears that share their activations (ragged row counts, a tail chunk with a partial step) in
+    ONE launch of the tiled kernel -- equal to the members' own tiled launches bit for bit, as separate results and
+    written side by side into one array; by the default rule (one launch beyond 32 rows, member by member below) against
+    the oracle; rows of no multiple of 128 elements go member by member, and cannot be written side by side by the op
+    itself (the wrapper joins them)."""
+    from any_precision_amd import _capi
+    for Ns, K in (((200, 64, 72), 1024), ((130, 130), 2176), ((64, 100, 40, 257), 4096)):
+        Ls = [make(N, K, seed=N + K + i) for i, N in enumerate(Ns)]
+        gpu = [layer_to_gpu(L) for L in Ls]
+        for b in (3, 4, 6, 8):
+            qs, ts = [q for q, _ in gpu], [luts[b] for _, luts in gpu]
+            for M in (17, 65, 200):
+                print(f"gemm group Ns={Ns} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                with _capi.tuning(gemm_tiled=2, gemm_tile_split=1):
+                    singles = [ext.gemm_kbit(xg, q, t, b) for q, t in zip(qs, ts)]
+                    outs = ext.gemm_kbit_group(xg, qs, ts, b)
+                    joint = ext.gemm_kbit_group(xg, qs, ts, b, concat=True)
+                for s_, o in zip(singles, outs):
+                    assert torch.equal(s_.view(torch.int16), o.view(torch.int16))
+                assert joint.shape == (M, sum(Ns)) and torch.equal(joint, torch.cat(singles, dim=-1))
+                outs = ext.gemm_kbit_group(xg, qs, ts, b)                  # default rule
+                for L, o in zip(Ls, outs):
+                    _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                    assert_close_gemv(o, want, f"group Ns={Ns} K={K} b={b} M={M} N={L.N}")
+    # K = 1056: the tiled kernel does not serve it
+    Ls = [make(N, 1056, seed=N) for N in (40, 24)]
+    gpu = [layer_to_gpu(L) for L in Ls]
+    x, xg = _x(50, 1056, seed=3)
+    qs, ts = [q for q, _ in gpu], [luts[5] for _, luts in gpu]
+    joint = ext.gemm_kbit_group(xg, qs, ts, 5, concat=True)
+    for L, o in zip(Ls, torch.split(joint, [40, 24], dim=-1)):
+        _, want = oracle.matmul_kbit(x, L.qweight, L.luts[5], 5, return_f64=True)
+        assert_close_gemv(o, want, f"group K=1056 N={L.N}")
+    out = torch.empty((50, 64), dtype=torch.float16, device="cuda")
+    rc = _capi.gemm_group(xg.data_ptr(), [q.data_ptr() for q in qs], [t.data_ptr() for t in ts],
+                          [out.data_ptr(), out.data_ptr() + 80], [40, 24], [64, 64], 50, 1056, 5, torch.cuda.current_stream().cuda_stream)
+    assert rc == _capi.AP_ESHAPE
+    q8, luts8 = layer_to_gpu(make(8, 64, seed=1))
+    with pytest.raises(ValueError, match="same in_features"):
+        ext.gemm_kbit_group(xg, [qs[0], q8], [ts[0], luts8[5]], 5)

@@ -128,3 +128,28 @@ def test_forward_takes_the_tiled_gemm_up_to_256_rows_at_3_and_4_bits(oracle):
         y = m(torch.from_numpy(x).cuda(), precision=b)
         _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
         assert_close_gemv(y, want, f"b={b} M={M}")
+
+
+def test_forward_group_beyond_32_rows_is_one_tiled_launch(oracle):
+    """Sets of linears on 33..256 rows go through gemm_kbit_group (one launch of the tiled kernel) where fused_set_pays
+    says so, with biases added afterwards; against the oracle, joined or as a list."""
+    from any_precision_amd.linear import forward_group, fused_set_pays
+    assert fused_set_pays(128, [4096, 4096, 4096], 3, 4096) and fused_set_pays(256, [11008, 11008], 5, 4096)
+    assert fused_set_pays(64, [11008, 11008], 8, 4096) and not fused_set_pays(128, [11008, 11008], 8, 4096)
+    assert fused_set_pays(128, [4096, 1024, 1024], 8, 4096) and not fused_set_pays(32, [4096, 4096], 3, 4096)
+    assert not fused_set_pays(257, [4096, 4096], 3, 4096) and not fused_set_pays(64, [4096, 4096], 3, 4000)
+    layers = [make(n, 256, seed=80 + n) for n in (4096, 512, 520)]
+    for bias in (False, True):
+        mods = [_module(L, bias=bias)[0] for L in layers]
+        for b, rows in ((3, 40), (8, 64), (5, 200), (8, 200)):
+            print(f"forward_group tiled bias={bias} b={b} rows={rows}", flush=True)
+            x = synth.make_x(rows, 256, seed=rows)
+            xg = torch.from_numpy(x).cuda()
+            outs = forward_group(mods, xg, b)
+            joined = forward_group(mods, xg, b, concat=True)
+            assert joined.shape == (rows, 5128) and torch.equal(joined, torch.cat(outs, dim=-1))
+            for L, m, got in zip(layers, mods, outs):
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                if bias:
+                    want = want + m.bias.double().cpu().numpy()
+                assert_close_gemv(got, want, f"forward_group tiled bias={bias} b={b} rows={rows} N={L.N}")
