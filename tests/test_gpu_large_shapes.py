@@ -39,7 +39,9 @@ def test_llama70b_mlp_shapes(N, K):
         got_w = ext.dequant_kbit(q, lut, b)
         assert torch.equal(got_w, want_w), f"dequant N={N} K={K} b={b}"
         del got_w
-        for M, fn in ((1, ext.matmul_kbit), (4, ext.matmul_kbit), (8, ext.matmul_kbit), (32, ext.gemm_kbit)):
+        # 200 and 520 rows: the tiled GEMM (tiles of 64 x 128 rows here, four and five of them along the activation rows)
+        for M, fn in ((1, ext.matmul_kbit), (4, ext.matmul_kbit), (8, ext.matmul_kbit), (32, ext.gemm_kbit), (200, ext.gemm_kbit),
+                      (520, ext.gemm_kbit)):
             x = torch.randn((M, K), device="cuda", generator=gen).half()
             want = x.double() @ want_w.double().T
             got = fn(x, q, lut, b).double()
@@ -51,7 +53,7 @@ def test_llama70b_mlp_shapes(N, K):
 def test_llama3_8b_mlp_shape_under_the_default_routing():
     """14336 x 4096 at M = 1..8 under the default routing: the dot-product kernel (1, 2 and part of
     3), the 4x4x4 matrix-core kernel with one (3, 4) and two (5..8) groups of activation rows; then the
-    fused GEMM at 16, 32 and 48 rows."""
+    fused GEMM at 16, 32 and 48 rows (K-split kernel up to 32, tiled kernel beyond) and at 100 and 300."""
     import any_precision_ext as ext
     N, K = 14336, 4096
     gen = torch.Generator(device="cuda")
@@ -69,7 +71,7 @@ def test_llama3_8b_mlp_shape_under_the_default_routing():
             assert (got - want).abs().max() <= REL_TOL * want.abs().max(), f"M={M} b={b}"
         # the fused GEMM under its default routing: two weight-row blocks per workgroup at up to 5 / 6
         # bits, chunks of 32 activation rows above 32
-        for M in (16, 32, 48):
+        for M in (16, 32, 48, 100, 300):
             print(f"llama3 mlp gemm b={b} M={M}", flush=True)
             x = torch.randn((M, K), device="cuda", generator=gen).half()
             want = x.double() @ want_w.T
