@@ -881,6 +881,42 @@ def routing_audit(args, torch, _capi, synth):
                     cases.append(case)
                     if us["default"] > 1.05 * us[best]:
                         losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
+            # the same sets through ap_gemm_kbit_group at 48 and 128 rows: the default against one launch of the tiled
+            # kernel and against a launch per member
+            for b in (bits if args.audit_gemm else ()):
+                for M in (48, 128):
+                    x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
+                    big = [torch.empty((M, N), dtype=torch.float16, device="cuda") for N in Ns]
+                    outs = arr(*[o.data_ptr() for o in big])
+
+                    def gemm_set(st):
+                        cur["j"] = (cur["j"] + 1) % pools[0].sets
+                        j = cur["j"]
+                        rc = lib.ap_gemm_kbit_group(x.data_ptr(), n, arr(*[P.qweight[j].data_ptr() for P in pools]),
+                                                    arr(*[P.luts[b][j].data_ptr() for P in pools]), outs, rows_arr, None, M, K, b, st)
+                        if rc != 0:
+                            raise RuntimeError(_capi.strerror(rc))
+
+                    def gemm_members(st):
+                        cur["j"] = (cur["j"] + 1) % pools[0].sets
+                        for P, o in zip(pools, big):
+                            rc = lib.ap_gemm_kbit(x.data_ptr(), P.qweight[cur["j"]].data_ptr(), P.luts[b][cur["j"]].data_ptr(),
+                                                  o.data_ptr(), M, P.N, K, b, st)
+                            if rc != 0:
+                                raise RuntimeError(_capi.strerror(rc))
+
+                    reps = min(pools[0].sets, 8)
+                    us = {"default": _graph_us(torch, side, gemm_set, reps), "launch_per_member": _graph_us(torch, side, gemm_members, reps)}
+                    if K % 128 == 0:
+                        with _capi.tuning(gemm_tiled=2):
+                            us["one_tiled_launch"] = _graph_us(torch, side, gemm_set, reps)
+                    us["default"] = min(us["default"], _graph_us(torch, side, gemm_set, reps))
+                    best = min((k for k in us if k != "default"), key=lambda k: us[k])
+                    case = {"entry": "ap_gemm_kbit_group", "N": list(Ns), "K": K, "w_bits": b, "M": M,
+                            "default_us": round(us["default"], 2), "best": best, "best_us": round(us[best], 2)}
+                    cases.append(case)
+                    if us["default"] > 1.05 * us[best]:
+                        losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
             del pools
             torch.cuda.empty_cache()
     within = 1 - len(losses) / len(cases)
@@ -889,7 +925,8 @@ def routing_audit(args, torch, _capi, synth):
         "value": round(within, 4), "unit": "fraction", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None,
         "data": "synthetic", "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate",
         "config": {"workload": f"linears of {args.audit_models} at {args.audit_rows} activation rows, w_bits 3, 4, 5, 8"
-                               + (", their q/k/v and gate/up sets" if args.audit_sets else "")
+                               + (", their q/k/v and gate/up sets" + (" (also through ap_gemm_kbit_group at 48 and 128 rows)" if args.audit_gemm else "")
+                                  if args.audit_sets else "")
                                + (", ap_gemm_kbit at 16, 32, 64, 128 rows" if args.audit_gemm else "")
                                + "; cold weight sets; HIP graphs; alternatives forced through ap_set_tuning"},
         "cases": len(cases), "worst_excess": max((l["excess"] for l in losses), default=0.0),
