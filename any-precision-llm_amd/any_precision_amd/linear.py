@@ -31,9 +31,10 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     shapes of the 7B / 8B / 13B / 70B layers at 48..256 activation rows) the fused form wins up to 256 rows:
     at 3 bits everywhere (4096 x 4096: 24-25 us against 39-43; 11008 x 4096: 41-57 against 58-73; 28672 x 8192 at 128
     rows: 118 against 201); at 4 bits up to 128 rows everywhere and up to 256 on linears of 4096 rows or of fewer than
-    8192 rows of at most 5120 elements (4096 x 4096: 26-27 against 39-45); at 5 and 6 bits up to 128 rows on linears of
+    8192 rows of at most 5120 elements (4096 x 4096: 24-25 against 39-45); at 5 and 6 bits up to 128 rows on linears of
     8192 rows or more (13824 x 5120: 71-73 against 74-80; 28672 x 8192: 153-160 against 214-223) and on those small
-    ones (5120 x 5120: 40-42 against 52), at 5 bits up to 256 on 4096 x 4096; at 7 and 8 bits up to 64 rows on wide
+    ones (5120 x 5120: 40-42 against 52), at 5 bits on the rest as well (4096 x 11008: 76 against 84) and up to 256 on
+    4096 x 4096 (32 against 41); at 7 and 8 bits up to 64 rows on wide
     linears (11008 x 4096: 41 against 53; 28672 x 8192: 139 against 232) and up to 128 on the small ones (5120 x 5120:
     48 against 52).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising the
     weight once."""
@@ -46,7 +47,8 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
             return True
         if w_bits == 4 and (rows <= 128 or out_features <= 4096 or small):
             return True
-        if w_bits in (5, 6) and ((rows <= 128 and (out_features >= 8192 or small)) or (w_bits == 5 and small and in_features <= 4096)):
+        if w_bits in (5, 6) and ((rows <= 128 and (w_bits == 5 or out_features >= 8192 or small))
+                                 or (w_bits == 5 and small and in_features <= 4096)):
             return True
         if w_bits >= 7 and ((rows <= 64 and wide) or (rows <= 128 and small)):
             return True

@@ -112,10 +112,13 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             xr[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + (size_t)(xrow[i] + koff));
         return valid;
     };
-    // units of words past the row end hold zeros
-    auto stage_store = [&](int buf, const u32x4(&xr)[MBW], bool valid) {
+    // units of words past the row end hold zeros (CHECK: the stage may have such units)
+    auto stage_store = [&](auto check_c, int buf, const u32x4(&xr)[MBW], bool valid) {
 #pragma unroll
-        for (int i = 0; i < MBW; i++) xt[kh][buf][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
+        for (int i = 0; i < MBW; i++) {
+            if constexpr (decltype(check_c)::value) xt[kh][buf][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
+            else xt[kh][buf][sr + 16 * i][su ^ sr] = xr[i];
+        }
     };
 
     // ---- prologue: planes of step 0, stage 0, tables
@@ -146,7 +149,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         const long long first = (long long)nb * (NC / 8), last = (long long)N * (NC / 8) - 1;
         for (int i = kh * NTHR + tid; i < TQ; i += KH * NTHR) dst[i] = src[min(first + i, last)];
     }
-    stage_store(0, xr[0], xvalid[0]);
+    stage_store(std::true_type{}, 0, xr[0], xvalid[0]);
     xvalid[1] = stage_load(step_at(0), active_at(0), 1, xr[1]);  // every row has at least four stages
     __syncthreads();
 
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         });
     };
     // words past the row end: zero weights (their activations are zeros too)
-    auto finish_b = [&](const uint32_t(&raw)[RB][NRAW], bool alive, half8_t(&b)[RB]) {
+    auto finish_b = [&](auto check_c, const uint32_t(&raw)[RB][NRAW], bool alive, half8_t(&b)[RB]) {
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
             u32x4 bw;
@@ -205,12 +208,16 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                 uint32_t packed;
                 if constexpr (PAIR) packed = raw[rb][i];
                 else packed = raw[rb][2 * i] | (raw[rb][2 * i + 1] << 16);
-                bw[i] = alive ? packed : 0u;
+                if constexpr (decltype(check_c)::value) bw[i] = alive ? packed : 0u;
+                else bw[i] = packed;
             }
             b[rb] = __builtin_bit_cast(half8_t, bw);
         }
     };
-    for (int it = 0; it < nit; it++) {
+    // One step.  CHECK: this step or the next (whose first stages are loaded and stored here) may reach past the end of
+    // the row or of this half's share; all other steps run without the selects that zero such words.
+    auto run_step = [&](auto check_c, int it) {
+        constexpr bool CHECK = decltype(check_c)::value;
         const int step = step_at(it), step_next = step_at(it + 1);
         const bool active = active_at(it), active_next = active_at(it + 1);
         const bool last = it + 1 == nit;
@@ -231,7 +238,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         const bool partial = 16 * (step + 1) > W;
         bool live[4];
 #pragma unroll
-        for (int wi = 0; wi < 4; wi++) live[wi] = active && (!partial || 16 * step + 4 * wi + grp < W);
+        for (int wi = 0; wi < 4; wi++) live[wi] = !CHECK || (active && (!partial || 16 * step + 4 * wi + grp < W));
 
         // One stage = byte group j of the 16 words: four octets (wi), each RB B operands and MBW A operands feeding
         // RB x MBW matrix instructions.  The LDS reads of octet wi + 1 (A operands, table entries) are issued before
@@ -249,7 +256,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             static_for<4>([&](auto wi_c) {
                 constexpr int wi = decltype(wi_c)::value, cur = wi & 1, nxt = cur ^ 1;
                 half8_t bfrag[RB];
-                finish_b(braw[cur], live[wi], bfrag);
+                finish_b(check_c, braw[cur], live[wi], bfrag);
                 if constexpr (wi < 3) {
                     issue_a(std::integral_constant<int, buf>{}, std::integral_constant<int, wi + 1>{}, afrag[nxt]);
                     issue_b(j_c, std::integral_constant<int, wi + 1>{}, braw[nxt]);
@@ -264,10 +271,20 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                         acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[cur][mb], bfrag[rb], acc[rb][mb], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             });
-            if (more) stage_store(buf ^ 1, xr[buf ^ 1], xvalid[buf ^ 1]);
+            if (more) stage_store(check_c, buf ^ 1, xr[buf ^ 1], xvalid[buf ^ 1]);
             // everyone is done with `buf`, and the other buffer is complete
             lds_only_barrier();
         });
+    };
+    // (tiles of 128 activation rows keep the one form with the selects: a second copy of the step costs them the
+    // registers of their second wave per SIMD -- 11008 x 4096 at 256 rows, 3 bits: 75 us against 59 -- while tiles of
+    // 64 gain 5-15 % from the copy without them)
+    for (int it = 0; it < nit; it++) {
+        const int s0 = kh * nit + it;  // this step and the next, before clamping
+        if (MBW > 4 || s0 + 1 >= steps || 16 * (s0 + 2) > W)
+            run_step(std::true_type{}, it);
+        else
+            run_step(std::false_type{}, it);
     }
 
     // D[i][j]: lane l holds activation rows i = 4 (l / 16) + v of the block and weight row j = l % 16

@@ -55,7 +55,8 @@ def test_fused_gemm_dispatch_rule():
     from any_precision_amd.linear import fused_gemm_pays
     assert all(fused_gemm_pays(m, n, b) for m in (9, 32) for n in (4096, 14336) for b in (3, 8))
     assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6) and fused_gemm_pays(64, 14336, 6, 8192)
-    assert not fused_gemm_pays(65, 4096, 5) and not fused_gemm_pays(65, 4096, 5, 11008) and not fused_gemm_pays(129, 4096, 6, 4096)
+    assert not fused_gemm_pays(65, 4096, 5) and fused_gemm_pays(65, 4096, 5, 11008) and not fused_gemm_pays(65, 4096, 6, 11008)
+    assert not fused_gemm_pays(129, 4096, 6, 4096)
     assert fused_gemm_pays(128, 4096, 8, 4096) and fused_gemm_pays(128, 11008, 5, 4096) and not fused_gemm_pays(128, 11008, 8, 4096)
     # the tiled kernel: 3 bits to 256 rows on linears of 4096 rows or more, 4 bits to 128, 4-5 bits to 256 on small linears,
     # 5-6 bits to 128 on linears of 8192 rows or more, every bit-width to 64 rows on wide linears
