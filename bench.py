@@ -1210,7 +1210,8 @@ def decode_tokens(args, torch, _capi, synth):
 
 def prefill_linears(args, torch, _capi, synth):
     """The seven linears of a Llama-2-7B layer on M = 32 x 512 activation rows through AnyPrecisionLinear's
-    large-batch branch: dequant_kbit to fp16, then the library GEMM.  Reports the share of the dequant."""
+    large-batch branch: dequant_kbit to fp16, then the library GEMM.  Reports the share of the dequant, and beside it
+    the same rows through ap_gemm_kbit (the tiled fused kernel, one launch per linear)."""
     from any_precision_amd import AnyPrecisionLinear
     import any_precision_ext as ext
     gen = torch.Generator(device="cuda")
@@ -1220,7 +1221,7 @@ def prefill_linears(args, torch, _capi, synth):
     rows = []
     with torch.inference_mode():
         for b in (3, 8):
-            t_total = t_deq = flops = 0.0
+            t_total = t_deq = t_fused = flops = 0.0
             for name, N, K in synth.LLAMA2_7B_LAYER:
                 lin = AnyPrecisionLinear(K, N, list(range(3, 9)), bias=False, device="cuda", dtype=torch.float16)
                 lin.qweight.copy_(torch.randint(-2**31, 2**31 - 1, lin.qweight.shape, dtype=torch.int32, device="cuda",
@@ -1242,10 +1243,13 @@ def prefill_linears(args, torch, _capi, synth):
                     return a0.elapsed_time(a1) / reps
                 t_total += run(lambda: lin(x, precision=b))
                 t_deq += run(lambda: ext.dequant_kbit(lin.qweight, lin._buffers[f"lut{b}"], b))
+                # the same rows through the fused tiled GEMM in one launch, for the record (it is not what the module uses here)
+                t_fused += run(lambda: ext.gemm_kbit(x, lin.qweight, lin._buffers[f"lut{b}"], b), reps=2)
                 flops += 2.0 * M * N * K
                 del lin, x
             rows.append({"w_bits": b, "ms_per_layer_linears": round(t_total, 3), "ms_dequant": round(t_deq, 3),
-                         "dequant_share": round(t_deq / t_total, 4), "TFLOPs": round(flops / t_total / 1e9, 1)})
+                         "dequant_share": round(t_deq / t_total, 4), "TFLOPs": round(flops / t_total / 1e9, 1),
+                         "fused_tiled_gemm_ms": round(t_fused, 3), "fused_tiled_gemm_TFLOPs": round(flops / t_fused / 1e9, 1)})
     print(json.dumps({
         "metric": "prefill linears TFLOP/s, Llama-2-7B layer set, 16384 activation rows",
         "value": round(sum(r["TFLOPs"] for r in rows) / len(rows), 1), "unit": "TFLOP/s", "n_gpus": 1,
