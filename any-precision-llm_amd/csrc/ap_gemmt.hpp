@@ -47,6 +47,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     __shared__ __attribute__((aligned(16))) uint8_t tables[BN][TB];
     __shared__ u32x4 xt[KH][2][BM][16];  // [K half][stage buffer][activation row][16-byte unit ^ (row & 15)]
     static_assert(KH == 1 || KH == 2, "");
+    static_assert(BN == 64, "the host numbers tiles of 64 weight rows through the members (GemmtMembers::tile0)");
     static_assert(KH == 1 || RB * MBW * 4 * kWave * kGemmtWaves * 4 <= (int)sizeof(xt) / KH, "partial tiles fit a half's stage buffers");
 
     const int lane = threadIdx.x;
