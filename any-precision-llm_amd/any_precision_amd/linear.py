@@ -29,7 +29,7 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).
     With the tiled kernel (rows of a multiple of 128 elements, linears of at least 4096 rows; measured on the linear
     shapes of the 7B / 8B / 13B / 70B layers at 48..256 activation rows) the fused form wins up to 256 rows:
-    at 3 bits everywhere (4096 x 4096: 24-25 us against 39-43; 11008 x 4096: 41-57 against 58-73; 28672 x 8192 at 128
+    at 3 bits everywhere (and up to 512 rows on linears of 4096 rows; 4096 x 4096: 22-23 us against 39-43; 11008 x 4096: 41-57 against 58-73; 28672 x 8192 at 128
     rows: 118 against 201); at 4 bits up to 128 rows everywhere and up to 256 on linears of 4096 rows or of fewer than
     8192 rows of at most 5120 elements (4096 x 4096: 24-25 against 39-45); at 5 and 6 bits up to 128 rows on linears of
     8192 rows or more (13824 x 5120: 71-73 against 74-80; 28672 x 8192: 153-160 against 214-223) and on those small
@@ -40,6 +40,8 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
+    if GEMM_MAX_M and w_bits == 3 and in_features > 0 and in_features % 128 == 0 and out_features == 4096 and rows <= 512:
+        return True         # 4096 x 4096 at 512 rows: 36 us against 44; 4096 x 11008: 94 against 100
     if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
         small = out_features < 8192 and in_features <= 5120
         wide = out_features > 10240 or (out_features >= 8192 and in_features <= 4096)

@@ -11,7 +11,9 @@
 //   * the activations of the tile are staged ONCE per workgroup in LDS, double-buffered, 256 contiguous bytes per row
 //     and stage (byte group j of the 16 words of a step: 128 consecutive elements), and every A operand a wave reads
 //     from there feeds RB matrix instructions; the 16-byte units of a row are XOR-swizzled with the row number so
-//     that the 16 rows of an operand read hit 16 different bank groups;
+//     that the 16 rows of an operand read hit 16 different bank groups.  While a stage is in work the next one is
+//     brought in by direct global -> LDS loads (no registers, no LDS store instructions); only stages that may reach
+//     past the end of a row go through registers, where the words past the end are zeroed;
 //   * accumulators (RB x MBW tiles of 16 x 16) stay in registers over the whole K loop: no K-split, no combine.
 // Per stage a wave issues 4 x RB x MBW matrix instructions between two barriers.  K must be a multiple of 128.
 // One launch serves up to four linears that share x (q/k/v, gate/up): their tiles of 64 weight rows are numbered through
@@ -45,10 +47,13 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     constexpr int BN = kGemmtWaves * WROWS, BM = 16 * MBW;
     constexpr int NTHR = kGemmtWaves * kWave;
     __shared__ __attribute__((aligned(16))) uint8_t tables[BN][TB];
-    __shared__ u32x4 xt[KH][2][BM][16];  // [K half][stage buffer][activation row][16-byte unit ^ (row & 15)]
+    // the two stage buffers, [K half][activation row][16-byte unit ^ (row & 15)] each: separate arrays, so that the
+    // compiler can tell the buffer a direct load fills from the one the matrix operands are read from (it waits for
+    // every outstanding direct load before an LDS read that may touch its destination)
+    __shared__ u32x4 xt0[KH][BM][16], xt1[KH][BM][16];
     static_assert(KH == 1 || KH == 2, "");
     static_assert(BN == 64, "the host numbers tiles of 64 weight rows through the members (GemmtMembers::tile0)");
-    static_assert(KH == 1 || RB * MBW * 4 * kWave * kGemmtWaves * 4 <= (int)sizeof(xt) / KH, "partial tiles fit a half's stage buffers");
+    static_assert(KH == 1 || RB * MBW * 4 * kWave * kGemmtWaves * 4 <= (int)sizeof(xt0) / KH, "partial tiles fit a half's stage buffer");
 
     const int lane = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.y);
@@ -102,6 +107,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     uint32_t xrow[MBW];                                     // byte offset of this thread's activation rows (past M: row M-1)
 #pragma unroll
     for (int i = 0; i < MBW; i++) xrow[i] = (uint32_t)min(m0 + sr + 16 * i, M - 1) * (uint32_t)K * 2u;
+    auto stage_buffer = [&](auto buf_c) -> u32x4(&)[KH][BM][16] {
+        if constexpr (decltype(buf_c)::value == 0) return xt0;
+        else return xt1;
+    };
     // returns whether this thread's unit lies inside the row (the loaded bytes are some valid ones otherwise)
     auto stage_load = [&](int step, bool active, int j, u32x4(&xr)[MBW]) {
         const int w0 = 16 * step, chunk = w0 >> 5;
@@ -114,21 +123,37 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         return valid;
     };
     // units of words past the row end hold zeros (CHECK: the stage may have such units)
-    auto stage_store = [&](auto check_c, int buf, const u32x4(&xr)[MBW], bool valid) {
+    auto stage_store = [&](auto check_c, auto buf_c, const u32x4(&xr)[MBW], bool valid) {
+        auto &xt = stage_buffer(buf_c);
 #pragma unroll
         for (int i = 0; i < MBW; i++) {
-            if constexpr (decltype(check_c)::value) xt[kh][buf][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
-            else xt[kh][buf][sr + 16 * i][su ^ sr] = xr[i];
+            if constexpr (decltype(check_c)::value) xt[kh][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
+            else xt[kh][sr + 16 * i][su ^ sr] = xr[i];
         }
+    };
+
+    // The same stage straight from global memory into LDS (no registers, no LDS store instruction): lane l of a wave
+    // writes the l-th 16-byte slot of the 1 KB that holds the wave's four rows, so it requests the unit that belongs
+    // there (slot = unit ^ row).  Only for stages that lie wholly inside the row: nothing can be zeroed on the way.
+    auto stage_dma = [&](int step, int j, auto buf_c) {
+        auto &xt = stage_buffer(buf_c);
+        const int w0 = 16 * step, chunk = w0 >> 5;
+        const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)((w0 & 31) + (su ^ sr)) << 4) +
+                              (uint32_t)j * (chunk == full_chunks ? tail_stride : 512u);
+#pragma unroll
+        for (int i = 0; i < MBW; i++)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(reinterpret_cast<const char *>(x) + (size_t)(xrow[i] + koff)),
+                (__attribute__((address_space(3))) void *)&xt[kh][16 * i + 4 * wv][0], 16, 0, 0);
     };
 
     // ---- prologue: planes of step 0, stage 0, tables
     uint32_t q[RB][BITS][4];
     fetch(step_at(0), q);
-    // stage t + 2 is requested while stage t is in work: slot t & 1 of xr carries stages t, t + 2, ...
-    u32x4 xr[2][MBW];
-    bool xvalid[2];
-    xvalid[0] = stage_load(step_at(0), active_at(0), 0, xr[0]);
+    // stage t + 1 is produced while stage t is in work: through registers where it may need zeros, else by the
+    // direct loads above
+    u32x4 xr[MBW];
+    bool xvalid = stage_load(step_at(0), active_at(0), 0, xr);
     if constexpr (PAIR) {
         // each wave builds pair tables of its own rows (with two K halves: its half of them), eight rows' loads in
         // flight at a time
@@ -150,14 +175,16 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         const long long first = (long long)nb * (NC / 8), last = (long long)N * (NC / 8) - 1;
         for (int i = kh * NTHR + tid; i < TQ; i += KH * NTHR) dst[i] = src[min(first + i, last)];
     }
-    stage_store(std::true_type{}, 0, xr[0], xvalid[0]);
-    xvalid[1] = stage_load(step_at(0), active_at(0), 1, xr[1]);  // every row has at least four stages
+    stage_store(std::true_type{}, std::integral_constant<int, 0>{}, xr, xvalid);
     __syncthreads();
 
     typedef __attribute__((address_space(3))) uint16_t lds_u16_t;
     typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
-    const uint32_t tab_base0 =
-        (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t *)&tables[0][0]) + (uint32_t)(wv * WROWS + col) * TB;
+    // table reads are written as offsets from the tables array (not as bare LDS addresses), so that the compiler knows
+    // they cannot touch a stage buffer a direct load is filling
+    typedef __attribute__((address_space(3))) uint8_t lds_u8_t;
+    const lds_u8_t *const tables_lds = (const lds_u8_t *)&tables[0][0];
+    const uint32_t tab_base0 = (uint32_t)(wv * WROWS + col) * TB;  // byte offset of this lane's row table
 
     float4_t acc[RB][MBW];
 #pragma unroll
@@ -172,9 +199,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     uint32_t braw[2][RB][NRAW];             // table entries of their B operands as they come from LDS
     // A operands of octet wi of the stage in buffer buf
     auto issue_a = [&](auto buf_c, auto wi_c, half8_t(&a)[MBW]) {
-        constexpr int buf = decltype(buf_c)::value, wi = decltype(wi_c)::value;
+        constexpr int wi = decltype(wi_c)::value;
+        auto &xt = stage_buffer(buf_c);
 #pragma unroll
-        for (int mb = 0; mb < MBW; mb++) a[mb] = __builtin_bit_cast(half8_t, xt[kh][buf][mb * 16 + col][(4 * wi + grp) ^ col]);
+        for (int mb = 0; mb < MBW; mb++) a[mb] = __builtin_bit_cast(half8_t, xt[kh][mb * 16 + col][(4 * wi + grp) ^ col]);
     };
     // table reads for the eight weights of byte group j of word wi of each row block
     auto issue_b = [&](auto j_c, auto wi_c, uint32_t(&raw)[RB][NRAW]) {
@@ -189,12 +217,12 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                     uint32_t a0;
                     if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
                     else a0 = tab_base + byte_offset<c, 2>(idx[wi][rb][i]);
-                    raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(a0);
+                    raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(tables_lds + a0);
                 } else {
                     uint32_t a0;
                     if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
                     else a0 = tab_base + byte_offset<c, 1>(idx[wi][rb][i]);
-                    raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(a0);
+                    raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(tables_lds + a0);
                 }
             });
         });
@@ -249,9 +277,11 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         // MBW KB of A operands and 4 x 4 x RB x 4..8 table reads against 4 x RB x MBW matrix instructions per wave).
         static_for<4>([&](auto j_c) {
             constexpr int j = decltype(j_c)::value, buf = j & 1;
-            const bool more = j < 3 || !last;     // a stage follows
-            const bool more2 = j < 2 || !last;    // two do
-            if (more2) xvalid[buf] = stage_load(j < 2 ? step : step_next, j < 2 ? active : active_next, (j + 2) & 3, xr[buf]);
+            const bool more = j < 3 || !last;     // a stage follows: it goes into the other buffer during this one
+            if (more) {
+                if constexpr (CHECK) xvalid = stage_load(j < 3 ? step : step_next, j < 3 ? active : active_next, (j + 1) & 3, xr);
+                else stage_dma(j < 3 ? step : step_next, (j + 1) & 3, std::integral_constant<int, buf ^ 1>{});
+            }
             issue_a(std::integral_constant<int, buf>{}, std::integral_constant<int, 0>{}, afrag[0]);
             if constexpr (j == 0) issue_b(j_c, std::integral_constant<int, 0>{}, braw[0]);
             static_for<4>([&](auto wi_c) {
@@ -272,17 +302,23 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                         acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[cur][mb], bfrag[rb], acc[rb][mb], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             });
-            if (more) stage_store(check_c, buf ^ 1, xr[buf ^ 1], xvalid[buf ^ 1]);
+            if constexpr (CHECK) {
+                if (more) stage_store(check_c, std::integral_constant<int, buf ^ 1>{}, xr, xvalid);
+            } else {
+                // the direct loads of the next stage (and everything requested before them) have landed:
+                // vmcnt(0), other counters untouched
+                if (more) __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
             // everyone is done with `buf`, and the other buffer is complete
             lds_only_barrier();
         });
     };
-    // (tiles of 128 activation rows keep the one form with the selects: a second copy of the step costs them the
-    // registers of their second wave per SIMD -- 11008 x 4096 at 256 rows, 3 bits: 75 us against 59 -- while tiles of
-    // 64 gain 5-15 % from the copy without them)
+    // (tiles of 128 activation rows at 5..7 bits keep the one form with the selects: the second copy of the step costs
+    // them the registers of their second wave per SIMD -- 11008 x 4096 at 256 rows, 5 bits: 91 us against 75; at 8 bits
+    // the tables leave room for one workgroup per CU either way)
     for (int it = 0; it < nit; it++) {
         const int s0 = kh * nit + it;  // this step and the next, before clamping
-        if (MBW > 4 || s0 + 1 >= steps || 16 * (s0 + 2) > W)
+        if ((MBW > 4 && BITS >= 5 && BITS <= 7) || s0 + 1 >= steps || 16 * (s0 + 2) > W)
             run_step(std::true_type{}, it);
         else
             run_step(std::false_type{}, it);
@@ -292,7 +328,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     if constexpr (KH == 2) {
         // the last barrier of the loop has passed: nobody reads the stage buffers any more.  Group 1 parks its tiles in
         // its own buffers, group 0 adds them to its own.
-        float *park = reinterpret_cast<float *>(&xt[1][0][0][0]) + wv * (RB * MBW * 4 * kWave);
+        float *park = reinterpret_cast<float *>(&xt0[1][0][0]) + wv * (RB * MBW * 4 * kWave);
         if (kh == 1) {
 #pragma unroll
             for (int rb = 0; rb < RB; rb++)

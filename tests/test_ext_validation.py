@@ -60,7 +60,8 @@ def test_fused_gemm_dispatch_rule():
     assert fused_gemm_pays(128, 4096, 8, 4096) and fused_gemm_pays(128, 11008, 5, 4096) and not fused_gemm_pays(128, 11008, 8, 4096)
     # the tiled kernel: 3 bits to 256 rows on linears of 4096 rows or more, 4 bits to 128, 4-5 bits to 256 on small linears,
     # 5-6 bits to 128 on linears of 8192 rows or more, every bit-width to 64 rows on wide linears
-    assert fused_gemm_pays(256, 11008, 3, 4096) and fused_gemm_pays(200, 4096, 3, 11008) and not fused_gemm_pays(257, 4096, 3, 4096)
+    assert fused_gemm_pays(256, 11008, 3, 4096) and fused_gemm_pays(200, 4096, 3, 11008) and not fused_gemm_pays(257, 5120, 3, 5120)
+    assert fused_gemm_pays(512, 4096, 3, 11008) and not fused_gemm_pays(513, 4096, 3, 4096) and not fused_gemm_pays(512, 4096, 4, 4096)
     assert not fused_gemm_pays(100, 1024, 3, 4096) and not fused_gemm_pays(200, 4096, 3, 4000)   # narrow; rows the tiled kernel does not take
     assert fused_gemm_pays(128, 11008, 4, 4096) and not fused_gemm_pays(192, 11008, 4, 4096) and fused_gemm_pays(256, 4096, 4, 4096)
     assert fused_gemm_pays(128, 4096, 4, 11008) and fused_gemm_pays(256, 4096, 4, 11008) and not fused_gemm_pays(129, 8192, 4, 8192)
