@@ -420,20 +420,20 @@ bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *
 
 // Where the tiled kernel is the fastest fused form (same sweep, and the linear shapes of the 7B / 8B / 13B / 70B layers
 // at 24..256 rows, against the K-split kernel, which serves more than 128 rows in chunks of 128): from 120 rows on
-// almost everywhere (4096 x 4096 at 128 rows: 24 / 26 / 33 us at 3 / 4 / 5 bits against 34-35; rows of more than 4096
+// everywhere (4096 x 4096 at 128 rows: 22 / 24 / 30 / 37 us at 3 / 4 / 5 / 8 bits against 34-36; rows of more than 4096
 // elements at 8 bits: 1.8-2x, e.g. 13824 x 5120 83 us against 171).  Its time does not depend on the number of
 // activation rows within a tile of 64, while the K-split kernel's grows with them and steps up beyond 32.  So wide
 // linears -- at least 8192 rows of at most 4096 elements, or more than 10240 rows of any length -- take it from 33
-// rows on (11008 x 4096 at 40 rows: 24-41 us against 32-44; 13824 x 5120: 31-53 against 49-76; 28672 x 8192 at 48 rows:
+// rows on (11008 x 4096 at 40 rows: 23-38 us against 32-44; 13824 x 5120: 31-53 against 49-76; 28672 x 8192 at 48 rows:
 // 75-135 against 122-216), at 7 and 8 bits on rows of more than 4096 elements from 24 (13824 x 5120: 54 against 65).
-// Linears of 5120..10240 rows of more than 4096 elements from 65 rows on (8192 x 8192 at 80 rows: 45-74 us against
-// 60-92; 5120 x 5120: 29-48 against 43-59); the rest (4096 rows) from 96 rows on at 3 and 4 bits.
+// Linears of 5120..10240 rows of more than 4096 elements from 48 rows on (8192 x 8192 at 64 rows: 38-64 us against
+// 43-76; 5120 x 5120: 26-44 against 32-49); the rest (up to 4096 rows) from 80 rows on at 3 and 4 bits, 104 at 5 and
+// 6, 120 at 7 and 8 (4096 x 4096 at 96 rows, 3 bits: 22 us against 26).
 bool gemmt_pays(int M, int N, int K, int w_bits) {
-    if (M > 128) return true;
+    if (M >= 120) return true;
     if ((N >= 8192 && K <= 4096) || N > 10240) return M > 32 || (K > 4096 && w_bits >= 7 && M >= 24);
-    if (N >= 5120 && K > 4096) return M > 64;
-    if (M >= 120) return w_bits <= 6 || N > 4096;  // 7-8 bits on up to 4096 rows: the K-split kernel is 6-9 % faster at 128 rows
-    return w_bits <= 4 && M >= 96;
+    if (N >= 5120 && K > 4096) return M >= 48;
+    return M >= (w_bits <= 4 ? 80 : (w_bits <= 6 ? 104 : 120));
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
