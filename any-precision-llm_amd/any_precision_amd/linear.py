@@ -33,10 +33,11 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     rows: 118 against 201); at 4 bits up to 128 rows everywhere and up to 256 on linears of 4096 rows or of fewer than
     8192 rows of at most 5120 elements (4096 x 4096: 24-25 against 39-45); at 5 and 6 bits up to 128 rows on linears of
     8192 rows or more (13824 x 5120: 71-73 against 74-80; 28672 x 8192: 153-160 against 214-223) and on those small
-    ones (5120 x 5120: 40-42 against 52), at 5 bits on the rest as well (4096 x 11008: 76 against 84) and up to 256 on
-    4096 x 4096 (32 against 41); at 7 and 8 bits up to 64 rows on wide
-    linears (11008 x 4096: 41 against 53; 28672 x 8192: 139 against 232) and up to 128 on the small ones (5120 x 5120:
-    48 against 52).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising the
+    ones (5120 x 5120: 40-42 against 52), at 5 bits on the rest as well and up to 256 on linears of 4096 rows
+    (4096 x 4096: 30 against 40; 4096 x 11008: 75 against 80); at 7 and 8 bits up to 64 rows on wide
+    linears (11008 x 4096: 36 against 55; 28672 x 8192: 139 against 232), up to 128 on the small ones (5120 x 5120:
+    48 against 52) and on linears of 4096 rows (4096 x 11008: 79 against 87), up to 256 on 4096 x 4096 (36 against
+    40).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising the
     weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
@@ -50,9 +51,10 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
         if w_bits == 4 and (rows <= 128 or out_features <= 4096 or small):
             return True
         if w_bits in (5, 6) and ((rows <= 128 and (w_bits == 5 or out_features >= 8192 or small))
-                                 or (w_bits == 5 and small and in_features <= 4096)):
+                                 or (w_bits == 5 and out_features <= 4096)):
             return True
-        if w_bits >= 7 and ((rows <= 64 and wide) or (rows <= 128 and small)):
+        if w_bits >= 7 and ((rows <= 64 and wide) or (rows <= 128 and (small or out_features <= 4096))
+                            or (out_features <= 4096 and in_features <= 4096)):
             return True
     if rows <= min(64, GEMM_MAX_M):
         if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):
@@ -64,13 +66,16 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
 def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bool:
     """Whether ONE launch of the tiled GEMM over linears that share their input (``gemm_kbit_group``) beats calling them
     one by one, each through whatever ``fused_gemm_pays`` picks (measured on the q/k/v and gate/up sets of the
-    Llama-2-7B / Llama-3-8B / 13B layers at 48..256 rows): from 33 rows on (below, the K-split kernel module by
-    module) up to 256 rows at up to 6 bits (q/k/v of the 7B layer at 128 rows, 3 bits: 39 us against 69 one by one and
+    Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 where every member has fewer than
+    8192 rows (q/k/v of the 7B layer at 16 rows, 3 bits: 16 us against 23; of the 13B layer: 20 against 36); wide
+    members (gate/up) at 9..32 rows are as fast module by module -- up to 256 rows at up to 6 bits (q/k/v of the 7B layer at 128 rows, 3 bits: 39 us against 69 one by one and
     129 for three dequant + GEMM pairs; gate/up at 256 rows, 5 bits: 125 against 146); at 7 and 8 bits up to 64 rows,
     and up to 128 where every member has fewer than 8192 rows (q/k/v at 8 bits: 66 against 127; gate/up: 129 against
     114 for the pairs)."""
-    if in_features % 128 or not 32 < rows <= 256 or sum(out_features) < 4096:
+    if in_features % 128 or not 8 < rows <= 256 or sum(out_features) < 4096:
         return False
+    if rows <= 32:
+        return max(out_features) < 8192 and in_features >= 1024
     return w_bits <= 6 or rows <= 64 or (rows <= 128 and max(out_features) < 8192)
 
 
@@ -79,7 +84,7 @@ def forward_group(modules, x, precision=None, concat=False):
     q/k/v or gate/up projections of a decoder layer); with ``concat`` the results joined along
     the last dimension.  Up to 8 activation rows and 4 modules they go through ``matmul_kbit_group``, which
     issues ONE launch wherever the dot-product kernel serves the set (always up to 4 rows; at 5..8 rows for
-    sets with narrow members and some 5-8-bit cases) and a launch per member otherwise; beyond 32 rows through
+    sets with narrow members and some 5-8-bit cases) and a launch per member otherwise; beyond 8 rows through
     ``gemm_kbit_group`` (one launch of the tiled GEMM) where the fused form pays for the set; else module by module.
     The reference has no counterpart (its ``fuse_layers`` is a stub, AnyPrecisionForCausalLM.py:168-172)."""
     rows = x.numel() // x.shape[-1]
@@ -87,8 +92,8 @@ def forward_group(modules, x, precision=None, concat=False):
     x = x.contiguous()
     K = modules[0].in_features
     same_input = 2 <= len(modules) <= 4 and all(m.in_features == K for m in modules)
-    # beyond 32 rows: one launch of the tiled GEMM (three 4096 x 4096 projections at 128 rows fill the chip that one of
-    # them leaves half idle); up to 32 rows the K-split kernel, module by module, is faster
+    # one launch of the tiled GEMM (three 4096 x 4096 projections at 128 rows fill the chip that one of them leaves half
+    # idle); up to 32 rows on wide members the K-split kernel, module by module, is as fast or faster
     tiled_set = same_input and fused_set_pays(rows, [m.out_features for m in modules], w_bits, K)
     if not same_input or (rows > 8 and not tiled_set):
         outs = [m(x, precision=w_bits) for m in modules]

@@ -45,7 +45,7 @@ enum {
     kGemmWalk,          // row-walking fused GEMM: 0 never, 1 where it pays, 2 wherever it fits
     kGemmWalkWgs,       // workgroups per CU its grid aims for
     kGemmTiled,         // tiled fused GEMM (ap_gemm_kbit): 0 never, 1 where it pays, 2 wherever it fits
-    kGemmTile,          // > 0: blocks of 16 activation rows in its tile, 4 or 8
+    kGemmTile,          // > 0: blocks of 16 activation rows in its tile: 1, 2, 4 or 8
     kGemmTileSplit,     // > 0: groups of four waves per workgroup of the 64-row tile, each on its share of K: 1 or 2
     kKnobCount
 };
@@ -405,35 +405,44 @@ bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *
     const long long small = tiles_n * ((M + 63) / 64);  // tiles of 64 x 64
     int mbw = 4;
     if (forced > 0) {
-        if (forced != 4 && forced != 8) return false;
+        if (forced != 1 && forced != 2 && forced != 4 && forced != 8) return false;
+        if (forced < 4 && K < 1024) return false;  // tiles of 16 and 32 rows exist in the two-half form only
         mbw = forced;
     } else if (M > 64) {
         if (10 * small >= (w_bits == 3 ? 30LL : 13LL) * cu_count()) mbw = 8;
     }
+    // A grid that leaves CUs idle takes the narrowest tile that still gives no CU a second workgroup: more workgroups
+    // dequantise the same weights, each for fewer activation rows (4096 x 4096 at 64 rows, 3 bits: 14 us with four
+    // times 64 tiles of 16 rows against 19 with 64 tiles of 64; at 128 rows 16 us with tiles of 32 against 19).
+    if (forced <= 0 && force_kh != 1 && mbw == 4 && K >= 1024) {
+        if (tiles_n * ((M + 15) / 16) <= cu_count()) mbw = 1;
+        else if (tiles_n * ((M + 31) / 32) <= cu_count()) mbw = 2;
+    }
     geo->mbw = mbw;
     // two K halves need at least two steps of 512 elements
-    geo->kh = mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && small <= cu_count())) ? 2 : 1;
+    geo->kh = mbw < 4 || (mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && small <= cu_count()))) ? 2 : 1;
     geo->grid_n = (int)tiles_n;  // tiles of 64 weight rows (of all linears of the launch)
     geo->grid_m = (M + 16 * mbw - 1) / (16 * mbw);
     return geo->grid_m <= 65535;
 }
 
 // Where the tiled kernel is the fastest fused form (same sweep, and the linear shapes of the 7B / 8B / 13B / 70B layers
-// at 24..256 rows, against the K-split kernel, which serves more than 128 rows in chunks of 128): from 120 rows on
-// everywhere (4096 x 4096 at 128 rows: 22 / 24 / 30 / 37 us at 3 / 4 / 5 / 8 bits against 34-36; rows of more than 4096
-// elements at 8 bits: 1.8-2x, e.g. 13824 x 5120 83 us against 171).  Its time does not depend on the number of
-// activation rows within a tile of 64, while the K-split kernel's grows with them and steps up beyond 32.  So wide
-// linears -- at least 8192 rows of at most 4096 elements, or more than 10240 rows of any length -- take it from 33
-// rows on (11008 x 4096 at 40 rows: 23-38 us against 32-44; 13824 x 5120: 31-53 against 49-76; 28672 x 8192 at 48 rows:
-// 75-135 against 122-216), at 7 and 8 bits on rows of more than 4096 elements from 24 (13824 x 5120: 54 against 65).
-// Linears of 5120..10240 rows of more than 4096 elements from 48 rows on (8192 x 8192 at 64 rows: 38-64 us against
-// 43-76; 5120 x 5120: 26-44 against 32-49); the rest (up to 4096 rows) from 80 rows on at 3 and 4 bits, 104 at 5 and
-// 6, 120 at 7 and 8 (4096 x 4096 at 96 rows, 3 bits: 22 us against 26).
+// at 16..256 rows, against the K-split kernel, which serves more than 128 rows in chunks of 128): from 104 rows on
+// everywhere (4096 x 4096 at 128 rows: 16 / 17 / 24 / 30 us at 3 / 4 / 5 / 8 bits against 33-35; rows of more than 4096
+// elements at 8 bits: 1.8-2x, e.g. 13824 x 5120 83 us against 171).  Its time grows with the activation rows in steps
+// of a tile (16, 32 or 64 rows, gemmt_geometry), while the K-split kernel's grows with every block of 16 rows and
+// steps up beyond 32.  So wide linears -- at least 8192 rows of at most 4096 elements, or more than 10240 rows of any
+// length -- take it from 33 rows on (11008 x 4096 at 48 rows: 20-36 us against 33-48; 28672 x 8192: 60-117 against
+// 122-216), and from 17 rows on up to 5 bits or on rows of more than 4096 elements (13824 x 5120 at 32 rows: 22-42 us
+// against 31-43; 14336 x 4096: 18-26 against 22-29).  Linears of 5120..10240 rows of more than 4096 elements from 33
+// rows on (5120 x 5120 at 48 rows: 18-36 us against 28-41); the rest (up to 4096 rows) from 33 rows on at 3 and 4 bits
+// (4096 x 4096 at 64 rows: 15-16 us against 19), from 65 at 5 bits and 81 at 6 (4096 x 4096 at 96 rows, 5 bits: 24 us
+// against 27), from 104 at 7 and 8 (a tie at 96).
 bool gemmt_pays(int M, int N, int K, int w_bits) {
-    if (M >= 120) return true;
-    if ((N >= 8192 && K <= 4096) || N > 10240) return M > 32 || (K > 4096 && w_bits >= 7 && M >= 24);
-    if (N >= 5120 && K > 4096) return M >= 48;
-    return M >= (w_bits <= 4 ? 80 : (w_bits <= 6 ? 104 : 120));
+    if (M >= 104) return true;
+    if ((N >= 8192 && K <= 4096) || N > 10240) return M > 32 || (M > 16 && (w_bits <= 5 || K > 4096));
+    if (N >= 5120 && K > 4096) return M > 32;
+    return M > (w_bits <= 4 ? 32 : (w_bits == 5 ? 64 : (w_bits == 6 ? 80 : 103)));
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
@@ -901,7 +910,7 @@ int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qwei
     if (!x || !qweight || !lut || !out || !N) return AP_ENULL;
     if (count < 1 || count > kGemmtMaxGroup) return AP_ELIMIT;
     if (M < 1) return AP_EBATCH;
-    long long tiles = 0, rows = 0;
+    long long tiles = 0, rows = 0;  // tiles of all members; rows of the largest
     bool strided = false;
     for (int g = 0; g < count; g++) {
         if (!qweight[g] || !lut[g] || !out[g]) return AP_ENULL;
@@ -911,7 +920,7 @@ int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qwei
         if (ldo && ldo[g] < N[g]) return AP_ESHAPE;
         strided = strided || (ldo && ldo[g] != N[g]);
         tiles += (N[g] + 63) / 64;
-        rows += N[g];
+        rows = N[g] > rows ? N[g] : rows;
     }
     if (!aligned16(x)) return AP_EALIGN;
     drain_stale_error();
@@ -921,9 +930,11 @@ int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qwei
     // Tiles of different members run side by side, and the launch costs about what its largest member alone would,
     // while the K-split kernel's launches add up: measured on the q/k/v and gate/up sets of the 7B / 8B / 13B layers at
     // 48..256 rows the one launch is 1.1-3x faster than the members one by one (q/k/v of the 7B layer at 128 rows,
-    // 3 bits: 39 us against 69; of the 13B layer at 64 rows: 31 against 94) wherever there are more than 32 rows.
-    const bool pays = M > 32;
-    (void)rows;
+    // 3 bits: 39 us against 69; of the 13B layer at 64 rows: 31 against 94) wherever there are more than 32 rows.  Sets
+    // whose members all have fewer than 8192 rows (q/k/v) take it from 9 rows on, in tiles of 16 or 32 activation
+    // rows (7B q/k/v at 16 rows: 16-24 us against 23-26 at 3-5 bits, a tie at 8; 13B: 20-43 against 36-71); wide
+    // members (gate/up) at 9..32 rows are as fast or faster one by one.
+    const bool pays = M > 32 || (M > 8 && rows < 8192 && K >= 1024);
     if (fits && (strided || (count > 1 && mode > 0 && (mode >= 2 || pays))))
         return run_gemmt(tgeo, x, count, qweight, lut, out, N, ldo, M, K, w_bits, static_cast<hipStream_t>(stream));
     if (strided) return AP_ESHAPE;  // only the tiled kernel writes rows that are not dense

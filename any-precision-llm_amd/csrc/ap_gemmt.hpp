@@ -16,6 +16,8 @@
 //     past the end of a row go through registers, where the words past the end are zeroed;
 //   * accumulators (RB x MBW tiles of 16 x 16) stay in registers over the whole K loop: no K-split, no combine.
 // Per stage a wave issues 4 x RB x MBW matrix instructions between two barriers.  K must be a multiple of 128.
+// MBW = 1 and 2 (tiles of 16 and 32 activation rows) are for grids that would leave CUs idle: the same weights are then
+// dequantised by several workgroups, each for fewer activation rows.
 // One launch serves up to four linears that share x (q/k/v, gate/up): their tiles of 64 weight rows are numbered through
 // (GemmtMembers), which fills the chip where one linear alone leaves CUs idle.
 #pragma once
@@ -263,7 +265,9 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                 else planes_to_indices<BITS, PRE>(qq, idx[wi][rb]);
             }
         }
-        if (!last) fetch(step_next, q);
+        if constexpr (CHECK) {
+            if (!last) fetch(step_next, q);
+        }
         const bool partial = 16 * (step + 1) > W;
         bool live[4];
 #pragma unroll
@@ -281,6 +285,15 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             if (more) {
                 if constexpr (CHECK) xvalid = stage_load(j < 3 ? step : step_next, j < 3 ? active : active_next, (j + 1) & 3, xr);
                 else stage_dma(j < 3 ? step : step_next, (j + 1) & 3, std::integral_constant<int, buf ^ 1>{});
+            }
+            if constexpr (!CHECK && j == 0) {
+                // the planes of the next step are requested AFTER the direct loads of the next stage: loads complete in
+                // order, so the wait for that stage at the end of this one can leave the planes in flight.  (After the
+                // last step this re-reads the planes of that step and uses nothing: a branch here would make the
+                // compiler wait for every load where the two paths join.)
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(step_next, q);
+                __builtin_amdgcn_sched_barrier(0);
             }
             issue_a(std::integral_constant<int, buf>{}, std::integral_constant<int, 0>{}, afrag[0]);
             if constexpr (j == 0) issue_b(j_c, std::integral_constant<int, 0>{}, braw[0]);
@@ -304,13 +317,17 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             });
             if constexpr (CHECK) {
                 if (more) stage_store(check_c, std::integral_constant<int, buf ^ 1>{}, xr, xvalid);
+                // everyone is done with `buf`, and the other buffer is complete
+                lds_only_barrier();
             } else {
-                // the direct loads of the next stage (and everything requested before them) have landed:
-                // vmcnt(0), other counters untouched
-                if (more) __builtin_amdgcn_s_waitcnt(0x0F70);
+                // The direct loads of the next stage (and everything requested before them) have landed, and this
+                // wave's LDS reads of `buf` are done: vmcnt(0 or the plane loads) lgkmcnt(0).  The bare barrier
+                // instruction, not the fenced form: the release fence makes the compiler wait for EVERY outstanding
+                // load here once direct loads are in flight, the planes included.
+                if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0x0070 | (BITS * RB));
+                else __builtin_amdgcn_s_waitcnt(0x0070);
+                __builtin_amdgcn_s_barrier();
             }
-            // everyone is done with `buf`, and the other buffer is complete
-            lds_only_barrier();
         });
     };
     // (tiles of 128 activation rows at 5..7 bits keep the one form with the selects: the second copy of the step costs

@@ -16,6 +16,10 @@ void launch_gemmt(const GemmtGeometry &geo, const uint16_t *x, const GemmtMember
     // LDS traffic per matrix instruction falls by less than a third)
     if (geo.mbw == 8)
         gemmt_kbit_kernel<BITS, 1, 8, 1><<<grid, block, 0, stream>>>(xh, members, M, K);
+    else if (geo.mbw == 1)
+        gemmt_kbit_kernel<BITS, 1, 1, 2><<<grid, block, 0, stream>>>(xh, members, M, K);
+    else if (geo.mbw == 2)
+        gemmt_kbit_kernel<BITS, 1, 2, 2><<<grid, block, 0, stream>>>(xh, members, M, K);
     else if (geo.kh == 2)
         gemmt_kbit_kernel<BITS, 1, 4, 2><<<grid, block, 0, stream>>>(xh, members, M, K);
     else

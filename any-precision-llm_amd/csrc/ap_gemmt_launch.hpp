@@ -9,8 +9,8 @@ namespace ap {
 constexpr int kGemmtWaves = 4;  // waves per workgroup, each on its own block(s) of 16 weight rows
 
 struct GemmtGeometry {
-    int mbw;     // blocks of 16 activation rows per workgroup tile (4 or 8); a workgroup owns 64 weight rows
-    int kh;      // groups of four waves per workgroup, each on its share of K (1, or 2 with mbw = 4)
+    int mbw;     // blocks of 16 activation rows per workgroup tile (1, 2, 4 or 8); a workgroup owns 64 weight rows
+    int kh;      // groups of four waves per workgroup, each on its share of K (2 with mbw < 4; 1 or 2 with mbw = 4; 1 with 8)
     int grid_n;  // tiles of 64 weight rows over all members: sum of ceil(N / 64)
     int grid_m;  // ceil(M / (16 mbw))
 };

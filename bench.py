@@ -55,7 +55,7 @@ def parse_args():
     ap.add_argument("--audit-models", default="7b,8b", help="routing_audit: comma list out of 7b, 8b, 13b, 70b")
     ap.add_argument("--audit-rows", default="1,2,3,4,5,8", help="routing_audit: activation row counts")
     ap.add_argument("--audit-sets", action="store_true", help="routing_audit: also the q/k/v and gate/up sets (ap_matmul_kbit_group)")
-    ap.add_argument("--audit-gemm", action="store_true", help="routing_audit: also ap_gemm_kbit at 16, 32, 64, 128 rows")
+    ap.add_argument("--audit-gemm", action="store_true", help="routing_audit: also ap_gemm_kbit at 16, 32, 48, 64, 96, 128 rows")
     ap.add_argument("--audit-decode", action="store_true",
                     help="llama2_7b_decode: instead of the sweep over w_bits, the decode graph re-recorded under each global "
                          "override of the GEMV launch rules (ap_set_tuning), tokens/s against the default rules'")
@@ -804,7 +804,7 @@ def routing_audit(args, torch, _capi, synth):
         # the fused GEMM of ap_gemm_kbit on the same weights: one or two row blocks per workgroup, the row-walking kernel,
         # the tiled kernel
         for b in bits:
-            for M in ((16, 32, 64, 128) if args.audit_gemm else ()):
+            for M in ((16, 32, 48, 64, 96, 128) if args.audit_gemm else ()):
                 x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
                 big_out = torch.empty((M, N), dtype=torch.float16, device="cuda")
 
@@ -820,7 +820,7 @@ def routing_audit(args, torch, _capi, synth):
                 for name, knobs in (("one_block", {"gemm_tiled": 0, "gemm_walk": 0, "gemm_rb2": 0}),
                                     ("two_blocks", {"gemm_tiled": 0, "gemm_walk": 0, "gemm_rb2": 2}),
                                     ("walking", {"gemm_tiled": 0, "gemm_walk": 2}), ("tiled", {"gemm_tiled": 2})):
-                    if name == "tiled" and (M < 48 or K % 128):
+                    if name == "tiled" and K % 128:
                         continue
                     with _capi.tuning(**knobs):
                         us[name] = _graph_us(torch, side, gemm, reps)
@@ -927,7 +927,7 @@ def routing_audit(args, torch, _capi, synth):
         "config": {"workload": f"linears of {args.audit_models} at {args.audit_rows} activation rows, w_bits 3, 4, 5, 8"
                                + (", their q/k/v and gate/up sets" + (" (also through ap_gemm_kbit_group at 48 and 128 rows)" if args.audit_gemm else "")
                                   if args.audit_sets else "")
-                               + (", ap_gemm_kbit at 16, 32, 64, 128 rows" if args.audit_gemm else "")
+                               + (", ap_gemm_kbit at 16, 32, 48, 64, 96, 128 rows" if args.audit_gemm else "")
                                + "; cold weight sets; HIP graphs; alternatives forced through ap_set_tuning"},
         "cases": len(cases), "worst_excess": max((l["excess"] for l in losses), default=0.0),
         "losses": sorted(losses, key=lambda l: -l["excess"]), "all_cases": cases}))

@@ -71,3 +71,6 @@ def test_fused_gemm_dispatch_rule():
     assert not fused_gemm_pays(64, 8192, 8, 8192) and fused_gemm_pays(128, 5120, 8, 5120) and not fused_gemm_pays(128, 5120, 6, 13824)
     assert fused_gemm_pays(64, 5120, 5, 13824) and not fused_gemm_pays(64, 5120, 8, 13824)      # long rows, 6 bits on
     assert fused_gemm_pays(64, 1024, 8, 4096) and not fused_gemm_pays(64, 1024, 5, 8192)        # narrow, long rows
+    # linears of 4096 rows: small grids take tiles of 16 or 32 activation rows, which moved their crossovers up
+    assert fused_gemm_pays(128, 4096, 8, 11008) and not fused_gemm_pays(129, 4096, 8, 11008) and fused_gemm_pays(256, 4096, 8, 4096)
+    assert fused_gemm_pays(256, 4096, 5, 11008) and not fused_gemm_pays(256, 4096, 6, 11008) and not fused_gemm_pays(257, 4096, 8, 4096)

@@ -197,8 +197,9 @@ def test_row_walking_kernel_on_a_wide_linear_by_default(ext, oracle):
 
 
 def test_tiled_kernel_agrees_with_the_oracle(ext, oracle):
-    """The tiled kernel (a workgroup owns 64 weight rows x 64 or 128 activation rows for the whole of K, activations
-    staged once per workgroup in LDS) forced with gemm_tiled = 2 and both tiles, on shapes small enough for the oracle:
+    """The tiled kernel (a workgroup owns 64 weight rows x 16, 32, 64 or 128 activation rows for the whole of K,
+    activations staged once per workgroup in LDS) forced with gemm_tiled = 2 and every tile, on shapes small enough for
+    the oracle:
     ragged row counts on both sides, one stage per byte group (K = 128), a tail chunk with a partial last step
     (K = 2176, 11008), several tiles of activation rows (M = 300).  Every output sums its products in the same order
     whatever the tile, so the two tiles agree bit for bit (with one group of waves per workgroup; with two, each on half
@@ -223,6 +224,12 @@ def test_tiled_kernel_agrees_with_the_oracle(ext, oracle):
                 with _capi.tuning(gemm_tiled=2, gemm_tile=4, gemm_tile_split=2):
                     halves = ext.gemm_kbit(xg, q, luts[b], b)
                 assert_close_gemv(halves, want, f"tiled halves N={N} K={K} b={b} M={M}")
+                # tiles of 16 and 32 activation rows (small grids; two halves of K always, so K >= 1024): the same sums
+                # in the same order as the two-half form of the 64-row tile
+                for tile in ((1, 2) if K >= 1024 else ()):
+                    with _capi.tuning(gemm_tiled=2, gemm_tile=tile):
+                        narrow = ext.gemm_kbit(xg, q, luts[b], b)
+                    assert torch.equal(narrow.view(torch.int16), halves.view(torch.int16)), (N, K, b, M, tile)
     # one-hot activation rows return columns of the dequantised weight exactly (K = 2176: also the partial step)
     N, K = 130, 2176
     L = make(N, K, seed=N + K)

@@ -132,12 +132,13 @@ def test_forward_takes_the_tiled_gemm_up_to_256_rows_at_3_and_4_bits(oracle):
 
 
 def test_forward_group_beyond_32_rows_is_one_tiled_launch(oracle):
-    """Sets of linears on 33..256 rows go through gemm_kbit_group (one launch of the tiled kernel) where fused_set_pays
+    """Sets of linears on 9..256 rows go through gemm_kbit_group (one launch of the tiled kernel) where fused_set_pays
     says so, with biases added afterwards; against the oracle, joined or as a list."""
     from any_precision_amd.linear import forward_group, fused_set_pays
     assert fused_set_pays(128, [4096, 4096, 4096], 3, 4096) and fused_set_pays(256, [11008, 11008], 5, 4096)
     assert fused_set_pays(64, [11008, 11008], 8, 4096) and not fused_set_pays(128, [11008, 11008], 8, 4096)
-    assert fused_set_pays(128, [4096, 1024, 1024], 8, 4096) and not fused_set_pays(32, [4096, 4096], 3, 4096)
+    assert fused_set_pays(128, [4096, 1024, 1024], 8, 4096) and fused_set_pays(9, [4096, 4096], 3, 4096)
+    assert not fused_set_pays(32, [11008, 11008], 3, 4096) and not fused_set_pays(8, [4096, 4096], 3, 4096)
     assert not fused_set_pays(257, [4096, 4096], 3, 4096) and not fused_set_pays(64, [4096, 4096], 3, 4000)
     layers = [make(n, 256, seed=80 + n) for n in (4096, 512, 520)]
     for bias in (False, True):
@@ -154,3 +155,13 @@ def test_forward_group_beyond_32_rows_is_one_tiled_launch(oracle):
                 if bias:
                     want = want + m.bias.double().cpu().numpy()
                 assert_close_gemv(got, want, f"forward_group tiled bias={bias} b={b} rows={rows} N={L.N}")
+    # 9..32 rows: sets whose members all have fewer than 8192 rows of at least 1024 elements (tiles of 16 or 32 rows)
+    layers = [make(n, 1024, seed=90 + n) for n in (4096, 200)]
+    mods = [_module(L, bias=False)[0] for L in layers]
+    for b, rows in ((3, 12), (6, 20), (8, 32)):
+        print(f"forward_group narrow tiles b={b} rows={rows}", flush=True)
+        x = synth.make_x(rows, 1024, seed=rows)
+        outs = forward_group(mods, torch.from_numpy(x).cuda(), b)
+        for L, got in zip(layers, outs):
+            _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+            assert_close_gemv(got, want, f"forward_group narrow tiles b={b} rows={rows} N={L.N}")

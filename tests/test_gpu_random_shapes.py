@@ -48,6 +48,10 @@ def test_random_shapes(oracle, seed):
             with _capi.tuning(gemm_tiled=2, gemm_tile=tile, gemm_tile_split=split):
                 got = ext.gemm_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
             assert_close_gemv(got, want, f"tiled {tile}/{split} N={N} K={K} b={b} M={M}")
+            if K >= 1024:   # tiles of 16 or 32 activation rows (what small grids take), case by case in turn
+                with _capi.tuning(gemm_tiled=2, gemm_tile=1 + (c & 1)):
+                    got = ext.gemm_kbit(torch.from_numpy(x).cuda(), q, luts[b], b)
+                assert_close_gemv(got, want, f"tiled {1 + (c & 1)} N={N} K={K} b={b} M={M}")
             M = int(rng2.integers(129, 300))
             print(f"random case {seed}/{c}: tiled default M={M}", flush=True)
             x = synth.make_x(M, K, seed=M + c)
