@@ -66,7 +66,7 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
 def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bool:
     """Whether ONE launch of the tiled GEMM over linears that share their input (``gemm_kbit_group``) beats calling them
     one by one, each through whatever ``fused_gemm_pays`` picks (measured on the q/k/v and gate/up sets of the
-    Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 where every member has fewer than
+    Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 (17 at 7 and 8 bits) where every member has fewer than
     8192 rows (q/k/v of the 7B layer at 16 rows, 3 bits: 16 us against 23; of the 13B layer: 20 against 36); wide
     members (gate/up) at 9..32 rows are as fast module by module -- up to 256 rows at up to 6 bits (q/k/v of the 7B layer at 128 rows, 3 bits: 39 us against 69 one by one and
     129 for three dequant + GEMM pairs; gate/up at 256 rows, 5 bits: 125 against 146); at 7 and 8 bits up to 64 rows,
@@ -75,7 +75,7 @@ def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bo
     if in_features % 128 or not 8 < rows <= 256 or sum(out_features) < 4096:
         return False
     if rows <= 32:
-        return max(out_features) < 8192 and in_features >= 1024
+        return max(out_features) < 8192 and in_features >= 1024 and (w_bits <= 6 or rows > 16)
     return w_bits <= 6 or rows <= 64 or (rows <= 128 and max(out_features) < 8192)
 
 

@@ -932,9 +932,10 @@ int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qwei
     // 48..256 rows the one launch is 1.1-3x faster than the members one by one (q/k/v of the 7B layer at 128 rows,
     // 3 bits: 39 us against 69; of the 13B layer at 64 rows: 31 against 94) wherever there are more than 32 rows.  Sets
     // whose members all have fewer than 8192 rows (q/k/v) take it from 9 rows on, in tiles of 16 or 32 activation
-    // rows (7B q/k/v at 16 rows: 16-24 us against 23-26 at 3-5 bits, a tie at 8; 13B: 20-43 against 36-71); wide
-    // members (gate/up) at 9..32 rows are as fast or faster one by one.
-    const bool pays = M > 32 || (M > 8 && rows < 8192 && K >= 1024);
+    // rows (7B q/k/v at 16 rows: 16-24 us against 23-26 at 3-5 bits; 13B: 20-43 against 36-71), at 7 and 8 bits from 17
+    // (7B at 16 rows, 8 bits: 33 us against 30 one by one); wide members (gate/up) at 9..32 rows are within 10 % either
+    // way one by one.
+    const bool pays = M > 32 || (M > (w_bits <= 6 ? 8 : 16) && rows < 8192 && K >= 1024);
     if (fits && (strided || (count > 1 && mode > 0 && (mode >= 2 || pays))))
         return run_gemmt(tgeo, x, count, qweight, lut, out, N, ldo, M, K, w_bits, static_cast<hipStream_t>(stream));
     if (strided) return AP_ESHAPE;  // only the tiled kernel writes rows that are not dense

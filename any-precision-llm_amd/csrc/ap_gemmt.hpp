@@ -49,6 +49,12 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     constexpr int BN = kGemmtWaves * WROWS, BM = 16 * MBW;
     constexpr int NTHR = kGemmtWaves * kWave;
     __shared__ __attribute__((aligned(16))) uint8_t tables[BN][TB];
+    // 3 bits, conflict-free form of the pair table: [wave][entry 0..63][slot 0..31] dwords, slot = 16 (lane / 16 & 1) +
+    // row: the 32 lanes the LDS serves per cycle (16 rows x 2) read 32 different banks whatever their entries are --
+    // against about 3.5 cycles for 32 random addresses in a table per row.  Two copies of every row's table (8 KB per
+    // wave instead of 4).
+    constexpr bool CF = BITS == 3 && RB == 1 && MBW <= 4;
+    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * 32 : 1];
     // the two stage buffers, [K half][activation row][16-byte unit ^ (row & 15)] each: separate arrays, so that the
     // compiler can tell the buffer a direct load fills from the one the matrix operands are read from (it waits for
     // every outstanding direct load before an LDS read that may touch its destination)
@@ -156,7 +162,22 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     // direct loads above
     u32x4 xr[MBW];
     bool xvalid = stage_load(step_at(0), active_at(0), 0, xr);
-    if constexpr (PAIR) {
+    if constexpr (CF) {
+        // lane = (row r, copy, upper half h of the entries): entry e = (f2 s2 f1 s1 f0 s0) holds (lut[f], lut[s]); h = f2,
+        // and with two K halves group kh writes the entries with s2 = kh.  A store covers two entries x 32 slots.
+        const int h = lane >> 5;
+        const u32x4 t = *reinterpret_cast<const u32x4 *>(lut + (size_t)min(n0 + (lane & 15), N - 1) * NC);
+        const uint32_t f01 = h ? t[2] : t[0], f23 = h ? t[3] : t[1];
+        const uint32_t F[4] = {f01 & 0xffffu, f01 >> 16, f23 & 0xffffu, f23 >> 16};
+        uint32_t *dst = cftab + wv * 2048 + h * 1024 + (lane & 31);
+        for (int s2 = (KH == 2 ? kh : 0); s2 < (KH == 2 ? kh + 1 : 2); s2++) {
+            const uint32_t s01 = s2 ? t[2] : t[0], s23 = s2 ? t[3] : t[1];
+            const uint32_t S[4] = {s01 << 16, s01 & 0xffff0000u, s23 << 16, s23 & 0xffff0000u};
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                dst[(16 * s2 + i) * 32] = F[((i >> 3) & 1) * 2 + ((i >> 1) & 1)] | S[((i >> 2) & 1) * 2 + (i & 1)];
+        }
+    } else if constexpr (PAIR) {
         // each wave builds pair tables of its own rows (with two K halves: its half of them), eight rows' loads in
         // flight at a time
         const PairLane<BITS> pl = pair_lane<BITS>(lane);
@@ -187,6 +208,8 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     typedef __attribute__((address_space(3))) uint8_t lds_u8_t;
     const lds_u8_t *const tables_lds = (const lds_u8_t *)&tables[0][0];
     const uint32_t tab_base0 = (uint32_t)(wv * WROWS + col) * TB;  // byte offset of this lane's row table
+    const lds_u8_t *const cftab_lds = (const lds_u8_t *)&cftab[0];
+    const uint32_t cf_base = (uint32_t)(wv * 2048 + (lane & 31)) * 4u;  // ... of this lane's slot of entry 0
 
     float4_t acc[RB][MBW];
 #pragma unroll
@@ -216,10 +239,15 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                 constexpr int i = decltype(e_c)::value;
                 if constexpr (PAIR) {
                     // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
-                    uint32_t a0;
-                    if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
-                    else a0 = tab_base + byte_offset<c, 2>(idx[wi][rb][i]);
-                    raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(tables_lds + a0);
+                    if constexpr (CF) {
+                        // the index byte is 4 x entry; an entry is 128 bytes
+                        raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(cftab_lds + (cf_base + byte_offset<c, 5>(idx[wi][rb][i])));
+                    } else {
+                        uint32_t a0;
+                        if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
+                        else a0 = tab_base + byte_offset<c, 2>(idx[wi][rb][i]);
+                        raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(tables_lds + a0);
+                    }
                 } else {
                     uint32_t a0;
                     if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);

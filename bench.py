@@ -881,10 +881,10 @@ def routing_audit(args, torch, _capi, synth):
                     cases.append(case)
                     if us["default"] > 1.05 * us[best]:
                         losses.append(dict(case, excess=round(us["default"] / us[best] - 1, 3)))
-            # the same sets through ap_gemm_kbit_group at 48 and 128 rows: the default against one launch of the tiled
-            # kernel and against a launch per member
+            # the same sets through ap_gemm_kbit_group at 16, 32, 48 and 128 rows: the default against one launch of the
+            # tiled kernel and against a launch per member
             for b in (bits if args.audit_gemm else ()):
-                for M in (48, 128):
+                for M in (16, 32, 48, 128):
                     x = torch.randn((M, K), device="cuda", generator=gen).to(torch.float16)
                     big = [torch.empty((M, N), dtype=torch.float16, device="cuda") for N in Ns]
                     outs = arr(*[o.data_ptr() for o in big])
@@ -925,7 +925,7 @@ def routing_audit(args, torch, _capi, synth):
         "value": round(within, 4), "unit": "fraction", "n_gpus": 1, "higher_is_better": True, "vs_baseline": None,
         "data": "synthetic", "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate",
         "config": {"workload": f"linears of {args.audit_models} at {args.audit_rows} activation rows, w_bits 3, 4, 5, 8"
-                               + (", their q/k/v and gate/up sets" + (" (also through ap_gemm_kbit_group at 48 and 128 rows)" if args.audit_gemm else "")
+                               + (", their q/k/v and gate/up sets" + (" (also through ap_gemm_kbit_group at 16, 32, 48 and 128 rows)" if args.audit_gemm else "")
                                   if args.audit_sets else "")
                                + (", ap_gemm_kbit at 16, 32, 48, 64, 96, 128 rows" if args.audit_gemm else "")
                                + "; cold weight sets; HIP graphs; alternatives forced through ap_set_tuning"},
