@@ -31,6 +31,9 @@
 
 namespace ap {
 
+// What a direct load fetches for a 16-byte unit that lies past the end of its row (or belongs to an idle iteration).
+__device__ const uint32_t kGemmtZeros[64] = {};
+
 // KH = 1 or 2 groups of four waves per workgroup; with 2, group kh walks half of K (steps kh * ceil(steps / 2) ..) on its
 // own stage buffers and the two partial tiles are added in LDS at the end (group 0's sum + group 1's, always in that
 // order).  Twice the waves per tile: for grids that leave CUs with one workgroup of four waves, where no pipe is busy
@@ -52,13 +55,25 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     // 3 bits, conflict-free form of the pair table: [wave][entry 0..63][slot 0..31] dwords, slot = 16 (lane / 16 & 1) +
     // row: the 32 lanes the LDS serves per cycle (16 rows x 2) read 32 different banks whatever their entries are --
     // against about 3.5 cycles for 32 random addresses in a table per row.  Two copies of every row's table (8 KB per
-    // wave instead of 4).
-    constexpr bool CF = BITS == 3 && RB == 1 && MBW <= 4;
-    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * 32 : 1];
-    // the two stage buffers, [K half][activation row][16-byte unit ^ (row & 15)] each: separate arrays, so that the
+    // wave instead of 4), so only the two-half form, which has a CU to itself, uses it (one group of waves per tile,
+    // 11008 x 4096 at 256 rows: 53 us against 51, with two workgroups per CU instead of three).
+    constexpr bool CF = BITS == 3 && RB == 1 && KH == 2;
+    // 5..8 bits, the same for the plain table: [wave][entry][slot] dwords with the fp16 entry in the low half; 128 bytes
+    // per entry up to 7 bits, 64 at 8 bits (one copy: the two lanes of a row that are served together collide when
+    // their entries differ, 2 cycles instead of 1 -- against 3.5).  16..64 KB per workgroup, so only the two-half
+    // form, which has a CU to itself, uses it.
+    constexpr bool CF16 = BITS >= 5 && RB == 1 && KH == 2;
+    constexpr int SLOTS = BITS == 8 ? 16 : 32;
+    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * 32 : (CF16 ? kGemmtWaves * NC * SLOTS : 1)];
+    // The stage buffers, [K half][activation row][16-byte unit ^ (row & 15)] each: separate arrays, so that the
     // compiler can tell the buffer a direct load fills from the one the matrix operands are read from (it waits for
-    // every outstanding direct load before an LDS read that may touch its destination)
+    // every outstanding direct load before an LDS read that may touch its destination).  Stage t of a group lives in
+    // buffer t % NBUF and is requested PD = NBUF - 1 stages before it is used: one stage ahead for tiles of 64 and 128
+    // rows, whose stages are long enough to cover the load, three for the narrow tiles (a stage of a 16-row tile is
+    // about 150 instructions per wave and used to wait for its successor's load every time).
+    constexpr int NBUF = MBW <= 2 ? 4 : 2, PD = NBUF - 1;
     __shared__ u32x4 xt0[KH][BM][16], xt1[KH][BM][16];
+    __shared__ u32x4 xt2[NBUF == 4 ? KH : 1][NBUF == 4 ? BM : 1][16], xt3[NBUF == 4 ? KH : 1][NBUF == 4 ? BM : 1][16];
     static_assert(KH == 1 || KH == 2, "");
     static_assert(BN == 64, "the host numbers tiles of 64 weight rows through the members (GemmtMembers::tile0)");
     static_assert(KH == 1 || RB * MBW * 4 * kWave * kGemmtWaves * 4 <= (int)sizeof(xt0) / KH, "partial tiles fit a half's stage buffer");
@@ -115,53 +130,42 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     uint32_t xrow[MBW];                                     // byte offset of this thread's activation rows (past M: row M-1)
 #pragma unroll
     for (int i = 0; i < MBW; i++) xrow[i] = (uint32_t)min(m0 + sr + 16 * i, M - 1) * (uint32_t)K * 2u;
-    auto stage_buffer = [&](auto buf_c) -> u32x4(&)[KH][BM][16] {
-        if constexpr (decltype(buf_c)::value == 0) return xt0;
-        else return xt1;
+    auto stage_buffer = [&](auto buf_c) -> auto & {
+        constexpr int buf = decltype(buf_c)::value;
+        if constexpr (buf == 0) return xt0;
+        else if constexpr (buf == 1) return xt1;
+        else if constexpr (buf == 2) return xt2;
+        else return xt3;
     };
-    // returns whether this thread's unit lies inside the row (the loaded bytes are some valid ones otherwise)
-    auto stage_load = [&](int step, bool active, int j, u32x4(&xr)[MBW]) {
-        const int w0 = 16 * step, chunk = w0 >> 5;
-        const bool valid = active && w0 + su < W;
-        const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)((w0 & 31) + (valid ? su : 0)) << 4) +
+
+    // A stage goes straight from global memory into LDS (no registers, no LDS store instruction): lane l of a wave
+    // writes the l-th 16-byte slot of the 1 KB that holds the wave's four rows, so it requests the unit that belongs
+    // there (slot = unit ^ row).  CHECK: the stage may have units of words past the end of the row, or belong to an
+    // iteration past the group's share of K; those units come from an array of zeros instead (nothing can be zeroed
+    // on the way).
+    const char *const zeros = reinterpret_cast<const char *>(kGemmtZeros) + 16 * su;
+    auto stage_dma = [&](auto check_c, int it_idx, int j, auto buf_c) {
+        auto &xt = stage_buffer(buf_c);
+        const int s = kh * nit + it_idx;  // the step, not clamped
+        const int w0 = 16 * s, chunk = w0 >> 5, u = su ^ sr;
+        const bool valid = !decltype(check_c)::value || (it_idx < nit && w0 + u < W);
+        const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)((w0 & 31) + u) << 4) +
                               (uint32_t)j * (chunk == full_chunks ? tail_stride : 512u);
 #pragma unroll
-        for (int i = 0; i < MBW; i++)
-            xr[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + (size_t)(xrow[i] + koff));
-        return valid;
-    };
-    // units of words past the row end hold zeros (CHECK: the stage may have such units)
-    auto stage_store = [&](auto check_c, auto buf_c, const u32x4(&xr)[MBW], bool valid) {
-        auto &xt = stage_buffer(buf_c);
-#pragma unroll
         for (int i = 0; i < MBW; i++) {
-            if constexpr (decltype(check_c)::value) xt[kh][sr + 16 * i][su ^ sr] = valid ? xr[i] : u32x4{0u, 0u, 0u, 0u};
-            else xt[kh][sr + 16 * i][su ^ sr] = xr[i];
+            const char *src = valid ? reinterpret_cast<const char *>(x) + (size_t)(xrow[i] + koff) : zeros;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                             (__attribute__((address_space(3))) void *)&xt[kh][16 * i + 4 * wv][0], 16, 0, 0);
         }
     };
 
-    // The same stage straight from global memory into LDS (no registers, no LDS store instruction): lane l of a wave
-    // writes the l-th 16-byte slot of the 1 KB that holds the wave's four rows, so it requests the unit that belongs
-    // there (slot = unit ^ row).  Only for stages that lie wholly inside the row: nothing can be zeroed on the way.
-    auto stage_dma = [&](int step, int j, auto buf_c) {
-        auto &xt = stage_buffer(buf_c);
-        const int w0 = 16 * step, chunk = w0 >> 5;
-        const uint32_t koff = ((uint32_t)chunk << 11) + ((uint32_t)((w0 & 31) + (su ^ sr)) << 4) +
-                              (uint32_t)j * (chunk == full_chunks ? tail_stride : 512u);
-#pragma unroll
-        for (int i = 0; i < MBW; i++)
-            __builtin_amdgcn_global_load_lds(
-                (const __attribute__((address_space(1))) void *)(reinterpret_cast<const char *>(x) + (size_t)(xrow[i] + koff)),
-                (__attribute__((address_space(3))) void *)&xt[kh][16 * i + 4 * wv][0], 16, 0, 0);
-    };
-
-    // ---- prologue: planes of step 0, stage 0, tables
+    // ---- prologue: planes of step 0, the first PD stages, tables
     uint32_t q[RB][BITS][4];
     fetch(step_at(0), q);
-    // stage t + 1 is produced while stage t is in work: through registers where it may need zeros, else by the
-    // direct loads above
-    u32x4 xr[MBW];
-    bool xvalid = stage_load(step_at(0), active_at(0), 0, xr);
+    static_for<PD>([&](auto t_c) {
+        constexpr int t = decltype(t_c)::value;
+        stage_dma(std::true_type{}, 0, t, std::integral_constant<int, t % NBUF>{});
+    });
     if constexpr (CF) {
         // lane = (row r, copy, upper half h of the entries): entry e = (f2 s2 f1 s1 f0 s0) holds (lut[f], lut[s]); h = f2,
         // and with two K halves group kh writes the entries with s2 = kh.  A store covers two entries x 32 slots.
@@ -177,6 +181,23 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             for (int i = 0; i < 16; i++)
                 dst[(16 * s2 + i) * 32] = F[((i >> 3) & 1) * 2 + ((i >> 1) & 1)] | S[((i >> 2) & 1) * 2 + (i & 1)];
         }
+    } else if constexpr (CF16) {
+        // lane = (row [, copy], part of the table); group kh copies its half of that part: 8 entries per 16-byte load,
+        // a store covers 64 / SLOTS entries x SLOTS slots
+        constexpr int PARTS = kWave / SLOTS, EPL = NC / PARTS / KH;
+        const int e0 = (lane / SLOTS) * (NC / PARTS) + kh * EPL;
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(lut + (size_t)min(n0 + (lane & 15), N - 1) * NC + e0);
+        uint32_t *dst = cftab + wv * (NC * SLOTS) + e0 * SLOTS + (lane % SLOTS);
+        u32x4 v[EPL / 8];
+#pragma unroll
+        for (int i = 0; i < EPL / 8; i++) v[i] = src[i];
+#pragma unroll
+        for (int i = 0; i < EPL / 8; i++)
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                dst[(8 * i + 2 * d) * SLOTS] = v[i][d] & 0xffffu;
+                dst[(8 * i + 2 * d + 1) * SLOTS] = v[i][d] >> 16;
+            }
     } else if constexpr (PAIR) {
         // each wave builds pair tables of its own rows (with two K halves: its half of them), eight rows' loads in
         // flight at a time
@@ -198,7 +219,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         const long long first = (long long)nb * (NC / 8), last = (long long)N * (NC / 8) - 1;
         for (int i = kh * NTHR + tid; i < TQ; i += KH * NTHR) dst[i] = src[min(first + i, last)];
     }
-    stage_store(std::true_type{}, std::integral_constant<int, 0>{}, xr, xvalid);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): the stages requested above are in LDS
     __syncthreads();
 
     typedef __attribute__((address_space(3))) uint16_t lds_u16_t;
@@ -209,7 +230,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     const lds_u8_t *const tables_lds = (const lds_u8_t *)&tables[0][0];
     const uint32_t tab_base0 = (uint32_t)(wv * WROWS + col) * TB;  // byte offset of this lane's row table
     const lds_u8_t *const cftab_lds = (const lds_u8_t *)&cftab[0];
-    const uint32_t cf_base = (uint32_t)(wv * 2048 + (lane & 31)) * 4u;  // ... of this lane's slot of entry 0
+    const uint32_t cf_base = (uint32_t)(wv * (CF16 ? NC * SLOTS : 2048) + lane % (CF16 ? SLOTS : 32)) * 4u;  // ... of this lane's slot of entry 0
 
     float4_t acc[RB][MBW];
 #pragma unroll
@@ -249,10 +270,15 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                         raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(tables_lds + a0);
                     }
                 } else {
-                    uint32_t a0;
-                    if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
-                    else a0 = tab_base + byte_offset<c, 1>(idx[wi][rb][i]);
-                    raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(tables_lds + a0);
+                    if constexpr (CF16) {
+                        // the index byte is 2 x entry and an entry 128 bytes; at 8 bits the entry, of 64 bytes
+                        raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(cftab_lds + (cf_base + byte_offset<c, 6>(idx[wi][rb][i])));
+                    } else {
+                        uint32_t a0;
+                        if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
+                        else a0 = tab_base + byte_offset<c, 1>(idx[wi][rb][i]);
+                        raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(tables_lds + a0);
+                    }
                 }
             });
         });
@@ -273,13 +299,13 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             b[rb] = __builtin_bit_cast(half8_t, bw);
         }
     };
-    // One step.  CHECK: this step or the next (whose first stages are loaded and stored here) may reach past the end of
-    // the row or of this half's share; all other steps run without the selects that zero such words.
+    // One step.  CHECK: this step or the next (whose first stages are requested here) may reach past the end of the row
+    // or of the walk; all other steps run without the selects that zero the weights of such words and that pick the
+    // source of a unit.
     auto run_step = [&](auto check_c, int it) {
         constexpr bool CHECK = decltype(check_c)::value;
         const int step = step_at(it), step_next = step_at(it + 1);
-        const bool active = active_at(it), active_next = active_at(it + 1);
-        const bool last = it + 1 == nit;
+        const bool active = active_at(it);
 #pragma unroll
         for (int rb = 0; rb < RB; rb++) {
 #pragma unroll
@@ -293,9 +319,6 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                 else planes_to_indices<BITS, PRE>(qq, idx[wi][rb]);
             }
         }
-        if constexpr (CHECK) {
-            if (!last) fetch(step_next, q);
-        }
         const bool partial = 16 * (step + 1) > W;
         bool live[4];
 #pragma unroll
@@ -304,21 +327,16 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         // One stage = byte group j of the 16 words: four octets (wi), each RB B operands and MBW A operands feeding
         // RB x MBW matrix instructions.  The LDS reads of octet wi + 1 (A operands, table entries) are issued before
         // the matrix instructions of octet wi; scheduling fences pin that order.  The table reads of the first octet
-        // of the next stage pass the barrier as well (the tables do not change).  Requesting the operands of a whole
-        // stage at once measured no faster: the LDS port, not its latency, bounds the stage (per stage and CU 4 x 4 x
-        // MBW KB of A operands and 4 x 4 x RB x 4..8 table reads against 4 x RB x MBW matrix instructions per wave).
+        // of the next stage pass the barrier as well (the tables do not change).
         static_for<4>([&](auto j_c) {
-            constexpr int j = decltype(j_c)::value, buf = j & 1;
-            const bool more = j < 3 || !last;     // a stage follows: it goes into the other buffer during this one
-            if (more) {
-                if constexpr (CHECK) xvalid = stage_load(j < 3 ? step : step_next, j < 3 ? active : active_next, (j + 1) & 3, xr);
-                else stage_dma(j < 3 ? step : step_next, (j + 1) & 3, std::integral_constant<int, buf ^ 1>{});
-            }
-            if constexpr (!CHECK && j == 0) {
-                // the planes of the next step are requested AFTER the direct loads of the next stage: loads complete in
-                // order, so the wait for that stage at the end of this one can leave the planes in flight.  (After the
-                // last step this re-reads the planes of that step and uses nothing: a branch here would make the
-                // compiler wait for every load where the two paths join.)
+            constexpr int j = decltype(j_c)::value, buf = j % NBUF;
+            // the stage PD ahead goes into the buffer that the stage before this one was read from (every wave has
+            // passed the barrier that ended it); past the end of the walk it fetches zeros that nobody reads
+            stage_dma(check_c, it + ((j + PD) >> 2), (j + PD) & 3, std::integral_constant<int, (j + PD) % NBUF>{});
+            if constexpr (j == 0) {
+                // the planes of the next step are requested AFTER the direct loads of this stage: loads complete in
+                // order, so the waits for stages below can leave the planes in flight.  (After the last step this
+                // re-reads the planes of that step and uses nothing: the waits below count on these loads.)
                 __builtin_amdgcn_sched_barrier(0);
                 fetch(step_next, q);
                 __builtin_amdgcn_sched_barrier(0);
@@ -343,19 +361,16 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                         acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag[cur][mb], bfrag[rb], acc[rb][mb], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             });
-            if constexpr (CHECK) {
-                if (more) stage_store(check_c, std::integral_constant<int, buf ^ 1>{}, xr, xvalid);
-                // everyone is done with `buf`, and the other buffer is complete
-                lds_only_barrier();
-            } else {
-                // The direct loads of the next stage (and everything requested before them) have landed, and this
-                // wave's LDS reads of `buf` are done: vmcnt(0 or the plane loads) lgkmcnt(0).  The bare barrier
-                // instruction, not the fenced form: the release fence makes the compiler wait for EVERY outstanding
-                // load here once direct loads are in flight, the planes included.
-                if constexpr (j == 0) __builtin_amdgcn_s_waitcnt(0x0070 | (BITS * RB));
-                else __builtin_amdgcn_s_waitcnt(0x0070);
-                __builtin_amdgcn_s_barrier();
-            }
+            // The next stage must have landed; it was requested PD - 1 stages before this one.  Loads complete in order,
+            // so what may stay outstanding is what was requested after it: the direct loads of the PD - 1 stages since
+            // (MBW each) and, up to stage PD - 1 of a step, the plane loads of the next step.  Then this wave's LDS reads
+            // of `buf` are done too (lgkmcnt(0)) and the workgroup meets.  The bare barrier instruction, not the fenced
+            // form: the release fence makes the compiler wait for EVERY outstanding load here once direct loads are in
+            // flight.
+            constexpr int keep = (PD - 1) * MBW + (j <= PD - 1 ? BITS * RB : 0);
+            static_assert(keep < 64, "");
+            __builtin_amdgcn_s_waitcnt(0x0070 | (keep & 15) | ((keep >> 4) << 14));
+            __builtin_amdgcn_s_barrier();
         });
     };
     // (tiles of 128 activation rows at 5..7 bits keep the one form with the selects: the second copy of the step costs
@@ -368,6 +383,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         else
             run_step(std::false_type{}, it);
     }
+    // the loads for stages past the end of the walk have landed too (they go where the partial tiles are parked below),
+    // for every wave
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    if constexpr (KH > 1) __syncthreads();
 
     // D[i][j]: lane l holds activation rows i = 4 (l / 16) + v of the block and weight row j = l % 16
     if constexpr (KH == 2) {
