@@ -34,9 +34,9 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     8192 rows of at most 5120 elements (4096 x 4096: 24-25 against 39-45); at 5 and 6 bits up to 128 rows on linears of
     8192 rows or more (13824 x 5120: 71-73 against 74-80; 28672 x 8192: 153-160 against 214-223) and on those small
     ones (5120 x 5120: 40-42 against 52), at 5 bits on the rest as well and up to 256 on linears of 4096 rows
-    (4096 x 4096: 30 against 40; 4096 x 11008: 75 against 80); at 7 and 8 bits up to 64 rows on wide
-    linears (11008 x 4096: 36 against 55; 28672 x 8192: 139 against 232), up to 128 on the small ones (5120 x 5120:
-    48 against 52) and on linears of 4096 rows (4096 x 11008: 79 against 87), up to 256 on 4096 x 4096 (36 against
+    (4096 x 4096: 30 against 40; 4096 x 11008: 75 against 80); at 7 and 8 bits up to 128 rows on wide
+    linears (11008 x 4096: 49 against 58; 28672 x 8192 at 64 rows: 139 against 232), on the small ones (5120 x 5120:
+    48 against 52) and on linears of 4096 rows (4096 x 11008: 72 against 87), up to 256 on 4096 x 4096 (36 against
     40).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising the
     weight once."""
     if rows <= min(32, GEMM_MAX_M):
@@ -53,7 +53,7 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
         if w_bits in (5, 6) and ((rows <= 128 and (w_bits == 5 or out_features >= 8192 or small))
                                  or (w_bits == 5 and out_features <= 4096)):
             return True
-        if w_bits >= 7 and ((rows <= 64 and wide) or (rows <= 128 and (small or out_features <= 4096))
+        if w_bits >= 7 and ((rows <= 128 and (wide or small or out_features <= 4096))
                             or (out_features <= 4096 and in_features <= 4096)):
             return True
     if rows <= min(64, GEMM_MAX_M):
@@ -66,7 +66,7 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
 def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bool:
     """Whether ONE launch of the tiled GEMM over linears that share their input (``gemm_kbit_group``) beats calling them
     one by one, each through whatever ``fused_gemm_pays`` picks (measured on the q/k/v and gate/up sets of the
-    Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 (17 at 7 and 8 bits) where every member has fewer than
+    Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 where every member has at most
     8192 rows (q/k/v of the 7B layer at 16 rows, 3 bits: 16 us against 23; of the 13B layer: 20 against 36); wide
     members (gate/up) at 9..32 rows are as fast module by module -- up to 256 rows at up to 6 bits (q/k/v of the 7B layer at 128 rows, 3 bits: 39 us against 69 one by one and
     129 for three dequant + GEMM pairs; gate/up at 256 rows, 5 bits: 125 against 146); at 7 and 8 bits up to 64 rows,
@@ -75,7 +75,7 @@ def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bo
     if in_features % 128 or not 8 < rows <= 256 or sum(out_features) < 4096:
         return False
     if rows <= 32:
-        return max(out_features) < 8192 and in_features >= 1024 and (w_bits <= 6 or rows > 16)
+        return max(out_features) <= 8192 and in_features >= 1024
     return w_bits <= 6 or rows <= 64 or (rows <= 128 and max(out_features) < 8192)
 
 

@@ -427,22 +427,22 @@ bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *
 }
 
 // Where the tiled kernel is the fastest fused form (same sweep, and the linear shapes of the 7B / 8B / 13B / 70B layers
-// at 16..256 rows, against the K-split kernel, which serves more than 128 rows in chunks of 128): from 104 rows on
-// everywhere (4096 x 4096 at 128 rows: 16 / 17 / 24 / 30 us at 3 / 4 / 5 / 8 bits against 33-35; rows of more than 4096
-// elements at 8 bits: 1.8-2x, e.g. 13824 x 5120 83 us against 171).  Its time grows with the activation rows in steps
-// of a tile (16, 32 or 64 rows, gemmt_geometry), while the K-split kernel's grows with every block of 16 rows and
-// steps up beyond 32.  So wide linears -- at least 8192 rows of at most 4096 elements, or more than 10240 rows of any
-// length -- take it from 33 rows on (11008 x 4096 at 48 rows: 20-36 us against 33-48; 28672 x 8192: 60-117 against
-// 122-216), and from 17 rows on up to 5 bits or on rows of more than 4096 elements (13824 x 5120 at 32 rows: 22-42 us
-// against 31-43; 14336 x 4096: 18-26 against 22-29).  Linears of 5120..10240 rows of more than 4096 elements from 33
-// rows on (5120 x 5120 at 48 rows: 18-36 us against 28-41); the rest (up to 4096 rows) from 33 rows on at 3 and 4 bits
-// (4096 x 4096 at 64 rows: 15-16 us against 19), from 65 at 5 bits and 81 at 6 (4096 x 4096 at 96 rows, 5 bits: 24 us
-// against 27), from 104 at 7 and 8 (a tie at 96).
+// at 16..256 rows, against the K-split kernel, which serves more than 128 rows in chunks of 128).  Its time grows with
+// the activation rows in steps of a tile (16, 32 or 64 rows, gemmt_geometry), while the K-split kernel's grows with
+// every block of 16 rows and steps up beyond 32 (4096 x 4096 at 128 rows: 15 / 19 / 22 / 29 us at 3 / 4 / 5 / 8 bits
+// against 34-36; rows of more than 4096 elements at 8 bits: 1.8-2x, e.g. 13824 x 5120 83 us against 171).  Wide linears
+// -- at least 8192 rows of at most 4096 elements, or more than 10240 rows of any length -- take it from 17 rows on
+// (11008 x 4096 at 48 rows: 20-36 us against 33-48; 14336 x 4096 at 32 rows: 18-33 against 22-36); those of at most
+// 16384 rows, whose grid has room for tiles of 16 activation rows, from 9 up to 4 bits or on rows of more than 4096
+// elements (11008 x 4096 at 16 rows, 3 bits: 12.8 us against 14.3; 13824 x 5120: 17-37 against 20-45; 28672 x 8192
+// at 16 rows would be 59-90 against 45-75).  Linears of 5120..10240 rows of more than 4096 elements from 33 rows on (5120 x 5120 at 48 rows:
+// 18-36 us against 28-41), from 17 at 3 bits (8192 x 8192 at 32 rows: 19.7 against 21.9); the rest (up to 4096 rows)
+// from 33 rows on at 3 and 4 bits (4096 x 4096 at 64 rows: 13-15 us against 19), from 49 at 5 bits (4096 x 11008 at 64
+// rows: 45 against 50), 65 at 6, 81 at 7 and 8 (4096 x 11008 at 96 rows, 8 bits: 68 against 75).
 bool gemmt_pays(int M, int N, int K, int w_bits) {
-    if (M >= 104) return true;
-    if ((N >= 8192 && K <= 4096) || N > 10240) return M > 32 || (M > 16 && (w_bits <= 5 || K > 4096));
-    if (N >= 5120 && K > 4096) return M > 32;
-    return M > (w_bits <= 4 ? 32 : (w_bits == 5 ? 64 : (w_bits == 6 ? 80 : 103)));
+    if ((N >= 8192 && K <= 4096) || N > 10240) return M > 16 || (M > 8 && N <= 16384 && (w_bits <= 4 || K > 4096));
+    if (N >= 5120 && K > 4096) return M > 32 || (M > 16 && w_bits == 3);
+    return M > (w_bits <= 4 ? 32 : (w_bits == 5 ? 48 : (w_bits == 6 ? 64 : 80)));
 }
 
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
@@ -932,10 +932,10 @@ int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qwei
     // 48..256 rows the one launch is 1.1-3x faster than the members one by one (q/k/v of the 7B layer at 128 rows,
     // 3 bits: 39 us against 69; of the 13B layer at 64 rows: 31 against 94) wherever there are more than 32 rows.  Sets
     // whose members all have fewer than 8192 rows (q/k/v) take it from 9 rows on, in tiles of 16 or 32 activation
-    // rows (7B q/k/v at 16 rows: 16-24 us against 23-26 at 3-5 bits; 13B: 20-43 against 36-71), at 7 and 8 bits from 17
-    // (7B at 16 rows, 8 bits: 33 us against 30 one by one); wide members (gate/up) at 9..32 rows are within 10 % either
-    // way one by one.
-    const bool pays = M > 32 || (M > (w_bits <= 6 ? 8 : 16) && rows < 8192 && K >= 1024);
+    // At 9..32 rows, sets whose members have at most 8192 rows (q/k/v) take it too, in tiles of 16 or 32 activation rows
+    // (7B q/k/v at 16 rows: 16-24 us against 23-26 at 3-5 bits; 13B: 20-40 against 36-68; 70B: 21-48 against 39-64); wide
+    // members (gate/up) are within 10 % either way one by one.
+    const bool pays = M > 32 || (M > 8 && rows <= 8192 && K >= 1024);
     if (fits && (strided || (count > 1 && mode > 0 && (mode >= 2 || pays))))
         return run_gemmt(tgeo, x, count, qweight, lut, out, N, ldo, M, K, w_bits, static_cast<hipStream_t>(stream));
     if (strided) return AP_ESHAPE;  // only the tiled kernel writes rows that are not dense

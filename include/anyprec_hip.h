@@ -90,7 +90,7 @@ int ap_matmul_kbit_swiglu(const uint16_t *x, const uint32_t *qweight_gate, const
  * M > 8 branch of AnyPrecisionLinear.forward (AnyPrecisionLinear.py:60-62: dequant_kbit,
  * main.cu:60-91, then torch.matmul) fused.  Two kernels: up to 128 activation rows a K-split
  * kernel with the weights of 16 rows in registers (more than 32 rows may run as launches of 32
- * each); from 104 rows on, and from 17..81 rows on where it measured faster, a tiled kernel whose
+ * each); from 81 rows on, and from 9..65 rows on where it measured faster, a tiled kernel whose
  * workgroups own 64 weight rows x 16..128 activation rows (the narrower the fewer tiles the grid
  * has) for the whole of K, ONE launch for any M (it needs K % 128 == 0; other row lengths go through the K-split kernel in chunks of 128 rows,
  * in order, on the same stream).  Correct for every M; faster than dequant + a library GEMM up to

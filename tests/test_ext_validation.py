@@ -57,7 +57,7 @@ def test_fused_gemm_dispatch_rule():
     assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6) and fused_gemm_pays(64, 14336, 6, 8192)
     assert not fused_gemm_pays(65, 4096, 5) and fused_gemm_pays(65, 4096, 5, 11008) and not fused_gemm_pays(65, 4096, 6, 11008)
     assert not fused_gemm_pays(129, 4096, 6, 4096)
-    assert fused_gemm_pays(128, 4096, 8, 4096) and fused_gemm_pays(128, 11008, 5, 4096) and not fused_gemm_pays(128, 11008, 8, 4096)
+    assert fused_gemm_pays(128, 4096, 8, 4096) and fused_gemm_pays(128, 11008, 5, 4096) and fused_gemm_pays(128, 11008, 8, 4096) and not fused_gemm_pays(129, 11008, 8, 4096)
     # the tiled kernel: 3 bits to 256 rows on linears of 4096 rows or more, 4 bits to 128, 4-5 bits to 256 on small linears,
     # 5-6 bits to 128 on linears of 8192 rows or more, every bit-width to 64 rows on wide linears
     assert fused_gemm_pays(256, 11008, 3, 4096) and fused_gemm_pays(200, 4096, 3, 11008) and not fused_gemm_pays(257, 5120, 3, 5120)
@@ -66,7 +66,7 @@ def test_fused_gemm_dispatch_rule():
     assert fused_gemm_pays(128, 11008, 4, 4096) and not fused_gemm_pays(192, 11008, 4, 4096) and fused_gemm_pays(256, 4096, 4, 4096)
     assert fused_gemm_pays(128, 4096, 4, 11008) and fused_gemm_pays(256, 4096, 4, 11008) and not fused_gemm_pays(129, 8192, 4, 8192)
     assert fused_gemm_pays(256, 4096, 5, 4096) and not fused_gemm_pays(256, 4096, 6, 4096) and not fused_gemm_pays(256, 5120, 5, 5120)
-    assert fused_gemm_pays(64, 14336, 8, 4096) and not fused_gemm_pays(64, 14336, 8, 4000) and not fused_gemm_pays(65, 14336, 8, 4096)
+    assert fused_gemm_pays(64, 14336, 8, 4096) and not fused_gemm_pays(64, 14336, 8, 4000) and fused_gemm_pays(65, 14336, 8, 4096)
     assert fused_gemm_pays(128, 28672, 6, 8192) and not fused_gemm_pays(129, 28672, 6, 8192) and fused_gemm_pays(64, 28672, 8, 8192)
     assert not fused_gemm_pays(64, 8192, 8, 8192) and fused_gemm_pays(128, 5120, 8, 5120) and not fused_gemm_pays(128, 5120, 6, 13824)
     assert fused_gemm_pays(64, 5120, 5, 13824) and not fused_gemm_pays(64, 5120, 8, 13824)      # long rows, 6 bits on
