@@ -64,7 +64,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     // form, which has a CU to itself, uses it.
     constexpr bool CF16 = BITS >= 5 && RB == 1 && KH == 2;
     constexpr int SLOTS = BITS == 8 ? 16 : 32;
-    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * 32 : (CF16 ? kGemmtWaves * NC * SLOTS : 1)];
+    // 4 bits, two-half form: the 256-entry pair table as [wave][entry][row] dwords, 64 bytes per entry and one copy
+    // (the same 64 KB as a table per row).
+    constexpr bool CF4 = BITS == 4 && RB == 1 && KH == 2;
+    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * 32 : (CF4 ? kGemmtWaves * 256 * 16 : (CF16 ? kGemmtWaves * NC * SLOTS : 1))];
     // The stage buffers, [K half][activation row][16-byte unit ^ (row & 15)] each: separate arrays, so that the
     // compiler can tell the buffer a direct load fills from the one the matrix operands are read from (it waits for
     // every outstanding direct load before an LDS read that may touch its destination).  Stage t of a group lives in
@@ -181,6 +184,26 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
             for (int i = 0; i < 16; i++)
                 dst[(16 * s2 + i) * 32] = F[((i >> 3) & 1) * 2 + ((i >> 1) & 1)] | S[((i >> 2) & 1) * 2 + (i & 1)];
         }
+    } else if constexpr (CF4) {
+        // entry e = (f3 s3 f2 s2 f1 s1 f0 s0) holds (lut[f], lut[s]).  lane = (row, f3, s3), the group of waves is f2: a
+        // lane writes the 32 entries (s2 f1 s1 f0 s0) of its eighth of the table from the halves of its row's values.
+        const int f3 = lane >> 5, s3 = (lane >> 4) & 1;
+        const u32x4 *row = reinterpret_cast<const u32x4 *>(lut + (size_t)min(n0 + (lane & 15), N - 1) * NC);
+        const u32x4 lo = row[0], hi = row[1];  // values 0..7, 8..15
+        const uint32_t fa = f3 ? (kh ? hi[2] : hi[0]) : (kh ? lo[2] : lo[0]);  // values 4 (2 f3 + f2) + {0, 1}
+        const uint32_t fb = f3 ? (kh ? hi[3] : hi[1]) : (kh ? lo[3] : lo[1]);  // ... + {2, 3}
+        const uint32_t F[4] = {fa & 0xffffu, fa >> 16, fb & 0xffffu, fb >> 16};
+        uint32_t S[8];                                                           // values 8 s3 + 0..7, in the high half
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t sv = s3 ? hi[k] : lo[k];
+            S[2 * k] = sv << 16;
+            S[2 * k + 1] = sv & 0xffff0000u;
+        }
+        uint32_t *dst = cftab + wv * (256 * 16) + ((f3 * 4 + s3 * 2 + kh) * 32) * 16 + (lane & 15);
+#pragma unroll
+        for (int i = 0; i < 32; i++)
+            dst[i * 16] = F[((i >> 3) & 1) * 2 + ((i >> 1) & 1)] | S[((i >> 4) & 1) * 4 + ((i >> 2) & 1) * 2 + (i & 1)];
     } else if constexpr (CF16) {
         // lane = (row [, copy], part of the table); group kh copies its half of that part: 8 entries per 16-byte load,
         // a store covers 64 / SLOTS entries x SLOTS slots
@@ -230,7 +253,8 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     const lds_u8_t *const tables_lds = (const lds_u8_t *)&tables[0][0];
     const uint32_t tab_base0 = (uint32_t)(wv * WROWS + col) * TB;  // byte offset of this lane's row table
     const lds_u8_t *const cftab_lds = (const lds_u8_t *)&cftab[0];
-    const uint32_t cf_base = (uint32_t)(wv * (CF16 ? NC * SLOTS : 2048) + lane % (CF16 ? SLOTS : 32)) * 4u;  // ... of this lane's slot of entry 0
+    const uint32_t cf_base = CF4 ? (uint32_t)(wv * (256 * 16) + (lane & 15)) * 4u
+                                 : (uint32_t)(wv * (CF16 ? NC * SLOTS : 2048) + lane % (CF16 ? SLOTS : 32)) * 4u;  // ... of this lane's slot of entry 0
 
     float4_t acc[RB][MBW];
 #pragma unroll
@@ -263,6 +287,9 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                     if constexpr (CF) {
                         // the index byte is 4 x entry; an entry is 128 bytes
                         raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(cftab_lds + (cf_base + byte_offset<c, 5>(idx[wi][rb][i])));
+                    } else if constexpr (CF4) {
+                        // the index byte is the entry, of 64 bytes
+                        raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(cftab_lds + (cf_base + byte_offset<c, 6>(idx[wi][rb][i])));
                     } else {
                         uint32_t a0;
                         if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
