@@ -101,8 +101,8 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
 
 /* ap_gemm_kbit for 1..4 linears that share x, K and w_bits (the q/k/v or gate/up projections of a decoder
  * layer on a batch of rows): out[g][M, N[g]] = x[M,K] . dequant(qweight[g], lut[g])^T.  Where the tiled
- * kernel serves the set (K % 128 == 0) and pays for it taken as one linear of all its rows, ONE launch
- * whose tiles of 64 weight rows run through the members -- three 4096 x 4096 projections at 128 rows fill
+ * kernel serves the set (K % 128 == 0) and pays -- more than 32 rows, or more than 8 where no member
+ * has more than 8192 rows -- ONE launch whose tiles of 64 weight rows run through the members -- three 4096 x 4096 projections at 128 rows fill
  * the chip that one of them leaves half idle; otherwise one ap_gemm_kbit per member, in order.
  * ldo (may be NULL: dense results) gives the distance in elements between consecutive rows of each
  * out[g], so that the results can be written side by side into one [M, sum N] array (out[g] = its
