@@ -52,22 +52,24 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     constexpr int BN = kGemmtWaves * WROWS, BM = 16 * MBW;
     constexpr int NTHR = kGemmtWaves * kWave;
     __shared__ __attribute__((aligned(16))) uint8_t tables[BN][TB];
-    // 3 bits, conflict-free form of the pair table: [wave][entry 0..63][slot 0..31] dwords, slot = 16 (lane / 16 & 1) +
-    // row: the 32 lanes the LDS serves per cycle (16 rows x 2) read 32 different banks whatever their entries are --
-    // against about 3.5 cycles for 32 random addresses in a table per row.  Two copies of every row's table (8 KB per
-    // wave instead of 4), so only the two-half form, which has a CU to itself, uses it (one group of waves per tile,
-    // 11008 x 4096 at 256 rows: 53 us against 51, with two workgroups per CU instead of three).
-    constexpr bool CF = BITS == 3 && RB == 1 && KH == 2;
-    // 5..8 bits, the same for the plain table: [wave][entry][slot] dwords with the fp16 entry in the low half; 128 bytes
-    // per entry up to 7 bits, 64 at 8 bits (one copy: the two lanes of a row that are served together collide when
-    // their entries differ, 2 cycles instead of 1 -- against 3.5).  16..64 KB per workgroup, so only the two-half
-    // form, which has a CU to itself, uses it.
-    constexpr bool CF16 = BITS >= 5 && RB == 1 && KH == 2;
-    constexpr int SLOTS = BITS == 8 ? 16 : 32;
-    // 4 bits, two-half form: the 256-entry pair table as [wave][entry][row] dwords, 64 bytes per entry and one copy
-    // (the same 64 KB as a table per row).
+    // Tables laid out by entry and slot, [wave][entry][slot] dwords: a table read is one random entry per lane, and with a
+    // table per row 32 random addresses cost the LDS about 3.5 cycles instead of 1.  Here the 32 lanes it serves per
+    // cycle -- 16 rows x 2 -- read by slot.  Two-half form (a CU to itself, LDS to spare): slot = 16 (lane / 16 & 1) +
+    // row, two copies of every row's table, 32 different banks whatever the entries.  One group of waves per tile
+    // (two or three workgroups share a CU): slot = row, one copy, the two lanes of a row collide when their entries
+    // differ (2 cycles), in the LDS a table per row would take or little more.
+    //   3 bits: the 64-entry pair table (8 or 4 KB per wave);
+    //   4 bits: two-half form the 256-entry pair table, one copy (the same 64 KB as a table per row); else the plain
+    //           table as below;
+    //   4..8 bits: the plain table with one fp16 entry per dword; two copies up to 7 bits in the two-half form
+    //           (16..64 KB per workgroup), one copy at 8 bits (64 KB) and with one group of waves (up to 6 bits there:
+    //           1..16 KB; the tables of 7 and 8 bits would cost a workgroup per CU).
+    constexpr bool CF = BITS == 3 && RB == 1;
     constexpr bool CF4 = BITS == 4 && RB == 1 && KH == 2;
-    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * 32 : (CF4 ? kGemmtWaves * 256 * 16 : (CF16 ? kGemmtWaves * NC * SLOTS : 1))];
+    constexpr bool CF16 = !PAIR && RB == 1 && (KH == 2 || BITS <= 6);
+    constexpr int SLOTS = (KH == 1 || BITS == 8) ? 16 : 32;
+    constexpr int ESHIFT = SLOTS == 32 ? 7 : 6;  // log2 of the bytes of an entry
+    __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * SLOTS : (CF4 ? kGemmtWaves * 256 * 16 : (CF16 ? kGemmtWaves * NC * SLOTS : 1))];
     // The stage buffers, [K half][activation row][16-byte unit ^ (row & 15)] each: separate arrays, so that the
     // compiler can tell the buffer a direct load fills from the one the matrix operands are read from (it waits for
     // every outstanding direct load before an LDS read that may touch its destination).  Stage t of a group lives in
@@ -170,20 +172,19 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
         stage_dma(std::true_type{}, 0, t, std::integral_constant<int, t % NBUF>{});
     });
     if constexpr (CF) {
-        // lane = (row r, copy, upper half h of the entries): entry e = (f2 s2 f1 s1 f0 s0) holds (lut[f], lut[s]); h = f2,
-        // and with two K halves group kh writes the entries with s2 = kh.  A store covers two entries x 32 slots.
-        const int h = lane >> 5;
+        // entry e = (f2 s2 f1 s1 f0 s0) holds (lut[f], lut[s]).  lane = (row, copy, f2) and the group of waves is s2 with two
+        // K halves, lane = (row, s2, f2) with one: a lane writes the 16 entries (f1 s1 f0 s0) of its quarter of the table
+        // from the halves of its row's eight values.
+        const int f2 = lane >> 5, s2 = KH == 2 ? kh : (lane >> 4) & 1;
         const u32x4 t = *reinterpret_cast<const u32x4 *>(lut + (size_t)min(n0 + (lane & 15), N - 1) * NC);
-        const uint32_t f01 = h ? t[2] : t[0], f23 = h ? t[3] : t[1];
+        const uint32_t f01 = f2 ? t[2] : t[0], f23 = f2 ? t[3] : t[1];
         const uint32_t F[4] = {f01 & 0xffffu, f01 >> 16, f23 & 0xffffu, f23 >> 16};
-        uint32_t *dst = cftab + wv * 2048 + h * 1024 + (lane & 31);
-        for (int s2 = (KH == 2 ? kh : 0); s2 < (KH == 2 ? kh + 1 : 2); s2++) {
-            const uint32_t s01 = s2 ? t[2] : t[0], s23 = s2 ? t[3] : t[1];
-            const uint32_t S[4] = {s01 << 16, s01 & 0xffff0000u, s23 << 16, s23 & 0xffff0000u};
+        const uint32_t s01 = s2 ? t[2] : t[0], s23 = s2 ? t[3] : t[1];
+        const uint32_t S[4] = {s01 << 16, s01 & 0xffff0000u, s23 << 16, s23 & 0xffff0000u};
+        uint32_t *dst = cftab + wv * (64 * SLOTS) + (32 * f2 + 16 * s2) * SLOTS + lane % SLOTS;
 #pragma unroll
-            for (int i = 0; i < 16; i++)
-                dst[(16 * s2 + i) * 32] = F[((i >> 3) & 1) * 2 + ((i >> 1) & 1)] | S[((i >> 2) & 1) * 2 + (i & 1)];
-        }
+        for (int i = 0; i < 16; i++)
+            dst[i * SLOTS] = F[((i >> 3) & 1) * 2 + ((i >> 1) & 1)] | S[((i >> 2) & 1) * 2 + (i & 1)];
     } else if constexpr (CF4) {
         // entry e = (f3 s3 f2 s2 f1 s1 f0 s0) holds (lut[f], lut[s]).  lane = (row, f3, s3), the group of waves is f2: a
         // lane writes the 32 entries (s2 f1 s1 f0 s0) of its eighth of the table from the halves of its row's values.
@@ -207,8 +208,10 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     } else if constexpr (CF16) {
         // lane = (row [, copy], part of the table); group kh copies its half of that part: 8 entries per 16-byte load,
         // a store covers 64 / SLOTS entries x SLOTS slots
-        constexpr int PARTS = kWave / SLOTS, EPL = NC / PARTS / KH;
-        const int e0 = (lane / SLOTS) * (NC / PARTS) + kh * EPL;
+        // (4 bits with one group: two parts of eight entries, written twice over)
+        constexpr int PARTS = (kWave / SLOTS) * KH * 8 <= NC ? kWave / SLOTS : NC / 8 / KH, EPL = NC / PARTS / KH;
+        static_assert(PARTS >= 1 && EPL % 8 == 0, "");
+        const int e0 = ((lane / SLOTS) % PARTS) * (NC / PARTS) + kh * EPL;
         const u32x4 *src = reinterpret_cast<const u32x4 *>(lut + (size_t)min(n0 + (lane & 15), N - 1) * NC + e0);
         uint32_t *dst = cftab + wv * (NC * SLOTS) + e0 * SLOTS + (lane % SLOTS);
         u32x4 v[EPL / 8];
@@ -254,7 +257,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     const uint32_t tab_base0 = (uint32_t)(wv * WROWS + col) * TB;  // byte offset of this lane's row table
     const lds_u8_t *const cftab_lds = (const lds_u8_t *)&cftab[0];
     const uint32_t cf_base = CF4 ? (uint32_t)(wv * (256 * 16) + (lane & 15)) * 4u
-                                 : (uint32_t)(wv * (CF16 ? NC * SLOTS : 2048) + lane % (CF16 ? SLOTS : 32)) * 4u;  // ... of this lane's slot of entry 0
+                                 : (uint32_t)(wv * ((CF16 ? NC : 64) * SLOTS) + lane % SLOTS) * 4u;  // ... of this lane's slot of entry 0
 
     float4_t acc[RB][MBW];
 #pragma unroll
@@ -285,8 +288,8 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                 if constexpr (PAIR) {
                     // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
                     if constexpr (CF) {
-                        // the index byte is 4 x entry; an entry is 128 bytes
-                        raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(cftab_lds + (cf_base + byte_offset<c, 5>(idx[wi][rb][i])));
+                        // the index byte is 4 x entry
+                        raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(cftab_lds + (cf_base + byte_offset<c, ESHIFT - 2>(idx[wi][rb][i])));
                     } else if constexpr (CF4) {
                         // the index byte is the entry, of 64 bytes
                         raw[rb][i] = *reinterpret_cast<const lds_u32_t *>(cftab_lds + (cf_base + byte_offset<c, 6>(idx[wi][rb][i])));
@@ -298,8 +301,8 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
                     }
                 } else {
                     if constexpr (CF16) {
-                        // the index byte is 2 x entry and an entry 128 bytes; at 8 bits the entry, of 64 bytes
-                        raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(cftab_lds + (cf_base + byte_offset<c, 6>(idx[wi][rb][i])));
+                        // the index byte is 2 x entry; at 8 bits the entry
+                        raw[rb][i] = *reinterpret_cast<const lds_u16_t *>(cftab_lds + (cf_base + byte_offset<c, ESHIFT - PRE>(idx[wi][rb][i])));
                     } else {
                         uint32_t a0;
                         if constexpr (PRE) a0 = byte_add<c>(tab_base, idx[wi][rb][i]);
