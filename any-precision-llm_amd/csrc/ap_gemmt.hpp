@@ -8,12 +8,14 @@
 //   * four waves, each on its own 16 RB weight rows; a wave rebuilds its weights in registers exactly as ap_gemm.hpp
 //     does (lane = row l % 16 and word 4s + l / 16; one B operand per byte group of a word) -- no LDS round trip and
 //     one table lookup per weight and tile of activation rows;
-//   * the activations of the tile are staged ONCE per workgroup in LDS, double-buffered, 256 contiguous bytes per row
-//     and stage (byte group j of the 16 words of a step: 128 consecutive elements), and every A operand a wave reads
-//     from there feeds RB matrix instructions; the 16-byte units of a row are XOR-swizzled with the row number so
-//     that the 16 rows of an operand read hit 16 different bank groups.  While a stage is in work the next one is
-//     brought in by direct global -> LDS loads (no registers, no LDS store instructions); only stages that may reach
-//     past the end of a row go through registers, where the words past the end are zeroed;
+//   * the activations of the tile are staged ONCE per workgroup in LDS, in two or four buffers, 256 contiguous bytes
+//     per row and stage (byte group j of the 16 words of a step: 128 consecutive elements), and every A operand a wave
+//     reads from there feeds RB matrix instructions; the 16-byte units of a row are XOR-swizzled with the row number so
+//     that the 16 rows of an operand read hit 16 different bank groups.  While a stage is in work the next one (or
+//     the third next) is brought in by direct global -> LDS loads (no registers, no LDS store instructions); units
+//     past the end of a row are fetched from an array of zeros;
+//   * the lookup tables sit in LDS by entry and slot where that fits, so that the lanes served together read
+//     different banks (below);
 //   * accumulators (RB x MBW tiles of 16 x 16) stay in registers over the whole K loop: no K-split, no combine.
 // Per stage a wave issues 4 x RB x MBW matrix instructions between two barriers.  K must be a multiple of 128.
 // MBW = 1 and 2 (tiles of 16 and 32 activation rows) are for grids that would leave CUs idle: the same weights are then
@@ -42,8 +44,8 @@ template <int BITS, int RB, int MBW, int KH>
 __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(const half_t *__restrict__ x, const GemmtMembers mem,
                                                                              int M, int K) {
     constexpr int NC = 1 << BITS;
-    // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 256 bytes per row): half the table reads,
-    // which are what loads the LDS port.  At 4 bits that table is 1 KB per row, 64 KB per workgroup: it pays where a CU
+    // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 64 dword entries per row): half the table
+    // reads, which are what loads the LDS port.  At 4 bits that table is 1 KB per row, 64 KB per workgroup: it pays where a CU
     // holds one workgroup anyway (the grids that run two K halves: 4096 x 4096 at 128 rows 26 us against 31) and costs
     // where it halves the workgroups per CU (11008 x 4096 at 256 rows: 92 us against 74), so only KH = 2 uses it.
     constexpr bool PAIR = BITS == 3 || (BITS == 4 && KH == 2);
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     const int nit = (steps + KH - 1) / KH;   // steps per K half; a half with one step fewer idles through the last
     // (all workgroups walk K in the same order: those in flight then read the same columns of the activations at
     // about the same time and share them in L2 -- walking from staggered starting steps measured 10-35 % slower)
-    // Iteration i of this half: its step, clamped into the row (an idle iteration loads valid bytes and uses none).
+    // Iteration i of this half: its step, clamped into the row (an idle iteration loads valid plane words and uses none).
     auto step_at = [&](int i) { return min(kh * nit + i, steps - 1); };
     auto active_at = [&](int i) { return kh * nit + i < steps; };
 
