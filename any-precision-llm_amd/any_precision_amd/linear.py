@@ -21,40 +21,35 @@ except ModuleNotFoundError:
 
 
 def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int = 0) -> bool:
-    """Whether the fused GEMM beats dequant_kbit + torch.matmul (measured on the 13 distinct linears of the
-    Llama-2-7B / Llama-3-8B / 13B / 70B layers at 3, 5, 8 bits): always up to 32 activation rows (1.3-4x at 16);
-    up to 64 on linears of fewer than 8192 rows, and on larger ones at up to 5 bits -- except, on rows of more
-    than 4096 elements, from 6 bits on linears of 5120 rows or more (5120 x 13824, 8 bits: 121 us against 86)
-    and from 5 bits on linears of at most 2048 rows (1024 x 8192); up to 128 on linears of 4096..8191
-    rows of at most 4096 elements (4096 x 4096: 33-35 us against 43; 1024 x 4096 at 96 rows: 25 against 18).
-    With the tiled kernel (rows of a multiple of 128 elements, linears of at least 4096 rows; measured on the linear
-    shapes of the 7B / 8B / 13B / 70B layers at 48..256 activation rows) the fused form wins up to 256 rows:
-    at 3 bits everywhere (and up to 512 rows on linears of 4096 rows; 4096 x 4096: 22-23 us against 39-43; 11008 x 4096: 41-57 against 58-73; 28672 x 8192 at 128
-    rows: 118 against 201); at 4 bits up to 128 rows everywhere and up to 256 on linears of 4096 rows or of fewer than
-    8192 rows of at most 5120 elements (4096 x 4096: 24-25 against 39-45); at 5 and 6 bits up to 128 rows on linears of
-    8192 rows or more (13824 x 5120: 71-73 against 74-80; 28672 x 8192: 153-160 against 214-223) and on those small
-    ones (5120 x 5120: 40-42 against 52), at 5 bits on the rest as well and up to 256 on linears of 4096 rows
-    (4096 x 4096: 30 against 40; 4096 x 11008: 75 against 80); at 7 and 8 bits up to 128 rows on wide
-    linears (11008 x 4096: 49 against 58; 28672 x 8192 at 64 rows: 139 against 232), on the small ones (5120 x 5120:
-    48 against 52) and on linears of 4096 rows (4096 x 11008: 72 against 87), up to 256 on 4096 x 4096 (36 against
-    40).  Beyond, one table lookup per weight and tile of activation rows costs more than materialising the
-    weight once."""
+    """Whether the fused GEMM beats dequant_kbit + torch.matmul.  Measured on the linear shapes of the Llama-2-7B /
+    Llama-3-8B / 13B / 70B layers at 96..512 activation rows and every bit-width (fused / pair, us):
+
+    * always up to 32 activation rows (1.3-4x at 16);
+    * rows of a multiple of 128 elements (the tiled kernel), linears of at least 4096 rows: up to 128 activation rows
+      at every bit-width (11008 x 4096, 8 bits: 50 / 58; 28672 x 8192: 189 / 234; 5120 x 13824: 93 / 113); up to 256
+      at up to 5 bits (11008 x 4096, 4 bits: 58 / 73; 13824 x 5120, 5 bits: 79 / 97), at 6 bits except on linears of
+      more than 16384 rows (28672 x 8192: 263 / 250), at 7 and 8 bits up to 192 on linears of at most 8192 rows
+      (8192 x 8192, 8 bits: 89 / 103; 11008 x 4096: 96 / 66) and up to 256 on 4096 x 4096 (33 / 39); up to 512 at
+      3 bits on linears of at most 8192 rows (4096 x 11008: 87 / 99; 8192 x 8192: 101 / 114; 14336 x 4096: 99 / 90);
+    * the same rows on linears of 1024..4095 rows: up to 512 activation rows at 3 and 4 bits (1024 x 4096: 11-15 /
+      18-23; at 6 bits and more the pair wins);
+    * other row lengths (the K-split kernel only): up to 64 on linears of fewer than 8192 rows, and on larger ones at up
+      to 5 bits -- except, on rows of more than 4096 elements, from 6 bits on linears of 5120 rows or more and from 5
+      bits on linears of at most 2048 rows; up to 128 on linears of 4096..8191 rows of at most 4096 elements.
+
+    Beyond, one table lookup per weight and tile of activation rows costs more than materialising the weight once."""
     if rows <= min(32, GEMM_MAX_M):
         return True
-    if GEMM_MAX_M and w_bits == 3 and in_features > 0 and in_features % 128 == 0 and out_features == 4096 and rows <= 512:
-        return True         # 4096 x 4096 at 512 rows: 36 us against 44; 4096 x 11008: 94 against 100
-    if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and out_features >= 4096 and rows <= 256:
-        small = out_features < 8192 and in_features <= 5120
-        wide = out_features > 10240 or (out_features >= 8192 and in_features <= 4096)
-        if w_bits == 3:
-            return True
-        if w_bits == 4 and (rows <= 128 or out_features <= 4096 or small):
-            return True
-        if w_bits in (5, 6) and ((rows <= 128 and (w_bits == 5 or out_features >= 8192 or small))
-                                 or (w_bits == 5 and out_features <= 4096)):
-            return True
-        if w_bits >= 7 and ((rows <= 128 and (wide or small or out_features <= 4096))
-                            or (out_features <= 4096 and in_features <= 4096)):
+    if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and rows <= 512:
+        if out_features >= 4096:
+            if rows <= 128:
+                return True
+            if rows <= 256:
+                if w_bits <= 6:
+                    return w_bits <= 5 or out_features <= 16384
+                return (rows <= 192 and out_features <= 8192) or (out_features <= 4096 and in_features <= 4096)
+            return w_bits == 3 and out_features <= 8192
+        if out_features >= 1024 and w_bits <= 4:
             return True
     if rows <= min(64, GEMM_MAX_M):
         if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):
@@ -68,15 +63,15 @@ def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bo
     one by one, each through whatever ``fused_gemm_pays`` picks (measured on the q/k/v and gate/up sets of the
     Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 where every member has at most
     8192 rows (q/k/v of the 7B layer at 16 rows, 3 bits: 16 us against 23; of the 13B layer: 20 against 36); wide
-    members (gate/up) at 9..32 rows are as fast module by module -- up to 256 rows at up to 6 bits (q/k/v of the 7B layer at 128 rows, 3 bits: 39 us against 69 one by one and
-    129 for three dequant + GEMM pairs; gate/up at 256 rows, 5 bits: 125 against 146); at 7 and 8 bits up to 64 rows,
-    and up to 128 where every member has fewer than 8192 rows (q/k/v at 8 bits: 66 against 127; gate/up: 129 against
-    114 for the pairs)."""
+    members (gate/up) at 9..32 rows are as fast module by module -- up to 128 rows at every bit-width (q/k/v of the 7B layer at 128 rows, 3 bits: 33 us against 44 one by one and
+    128 for three dequant + GEMM pairs; gate/up at 8 bits: 96 against 115 for the pairs), up to 256 at up to 6 bits
+    (gate/up at 5 bits: 105 against 145) and, at 7 and 8 bits, where every member has fewer than 8192 rows (q/k/v at 8
+    bits: 94 against 114; gate/up: 145 against 149)."""
     if in_features % 128 or not 8 < rows <= 256 or sum(out_features) < 4096:
         return False
     if rows <= 32:
         return max(out_features) <= 8192 and in_features >= 1024
-    return w_bits <= 6 or rows <= 64 or (rows <= 128 and max(out_features) < 8192)
+    return rows <= 128 or w_bits <= 6 or max(out_features) < 8192
 
 
 def forward_group(modules, x, precision=None, concat=False):

@@ -49,28 +49,25 @@ def test_cpu_tensors_are_rejected_not_computed():
 
 
 def test_fused_gemm_dispatch_rule():
-    """AnyPrecisionLinear sends 9..32 rows to the fused GEMM always, 33..64 only to small linears or
-    at up to 5 bits, more never (the reference sends everything above 8 rows to dequant + matmul,
-    AnyPrecisionLinear.py:60-62)."""
+    """Where AnyPrecisionLinear takes the fused GEMM instead of dequant + matmul (the reference sends everything above
+    8 rows to dequant + matmul, AnyPrecisionLinear.py:60-62): the rule as it was fitted to the measured sweep."""
     from any_precision_amd.linear import fused_gemm_pays
     assert all(fused_gemm_pays(m, n, b) for m in (9, 32) for n in (4096, 14336) for b in (3, 8))
-    assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6) and fused_gemm_pays(64, 14336, 6, 8192)
-    assert not fused_gemm_pays(65, 4096, 5) and fused_gemm_pays(65, 4096, 5, 11008) and not fused_gemm_pays(65, 4096, 6, 11008)
-    assert not fused_gemm_pays(129, 4096, 6, 4096)
-    assert fused_gemm_pays(128, 4096, 8, 4096) and fused_gemm_pays(128, 11008, 5, 4096) and fused_gemm_pays(128, 11008, 8, 4096) and not fused_gemm_pays(129, 11008, 8, 4096)
-    # the tiled kernel: 3 bits to 256 rows on linears of 4096 rows or more, 4 bits to 128, 4-5 bits to 256 on small linears,
-    # 5-6 bits to 128 on linears of 8192 rows or more, every bit-width to 64 rows on wide linears
-    assert fused_gemm_pays(256, 11008, 3, 4096) and fused_gemm_pays(200, 4096, 3, 11008) and not fused_gemm_pays(257, 5120, 3, 5120)
-    assert fused_gemm_pays(512, 4096, 3, 11008) and not fused_gemm_pays(513, 4096, 3, 4096) and not fused_gemm_pays(512, 4096, 4, 4096)
-    assert not fused_gemm_pays(100, 1024, 3, 4096) and not fused_gemm_pays(200, 4096, 3, 4000)   # narrow; rows the tiled kernel does not take
-    assert fused_gemm_pays(128, 11008, 4, 4096) and not fused_gemm_pays(192, 11008, 4, 4096) and fused_gemm_pays(256, 4096, 4, 4096)
-    assert fused_gemm_pays(128, 4096, 4, 11008) and fused_gemm_pays(256, 4096, 4, 11008) and not fused_gemm_pays(129, 8192, 4, 8192)
-    assert fused_gemm_pays(256, 4096, 5, 4096) and not fused_gemm_pays(256, 4096, 6, 4096) and not fused_gemm_pays(256, 5120, 5, 5120)
-    assert fused_gemm_pays(64, 14336, 8, 4096) and not fused_gemm_pays(64, 14336, 8, 4000) and fused_gemm_pays(65, 14336, 8, 4096)
-    assert fused_gemm_pays(128, 28672, 6, 8192) and not fused_gemm_pays(129, 28672, 6, 8192) and fused_gemm_pays(64, 28672, 8, 8192)
-    assert not fused_gemm_pays(64, 8192, 8, 8192) and fused_gemm_pays(128, 5120, 8, 5120) and not fused_gemm_pays(128, 5120, 6, 13824)
-    assert fused_gemm_pays(64, 5120, 5, 13824) and not fused_gemm_pays(64, 5120, 8, 13824)      # long rows, 6 bits on
+    # rows the tiled kernel does not take (not a multiple of 128 elements, or unknown): the K-split kernel's crossovers
+    assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6)
+    assert not fused_gemm_pays(65, 4096, 5) and not fused_gemm_pays(129, 4096, 6, 4000) and fused_gemm_pays(128, 4096, 6, 4000)
+    assert not fused_gemm_pays(64, 14336, 8, 4000) and not fused_gemm_pays(200, 4096, 3, 4000)
     assert fused_gemm_pays(64, 1024, 8, 4096) and not fused_gemm_pays(64, 1024, 5, 8192)        # narrow, long rows
-    # linears of 4096 rows: small grids take tiles of 16 or 32 activation rows, which moved their crossovers up
-    assert fused_gemm_pays(128, 4096, 8, 11008) and not fused_gemm_pays(129, 4096, 8, 11008) and fused_gemm_pays(256, 4096, 8, 4096)
-    assert fused_gemm_pays(256, 4096, 5, 11008) and not fused_gemm_pays(256, 4096, 6, 11008) and not fused_gemm_pays(257, 4096, 8, 4096)
+    # the tiled kernel, linears of at least 4096 rows: every bit-width up to 128 activation rows
+    assert all(fused_gemm_pays(128, n, b, k) for b in (3, 8) for n, k in ((4096, 4096), (11008, 4096), (5120, 13824), (28672, 8192)))
+    assert fused_gemm_pays(65, 14336, 8, 4096) and fused_gemm_pays(64, 5120, 8, 13824) and fused_gemm_pays(64, 8192, 8, 8192)
+    # up to 256 at up to 5 bits; at 6 bits except beyond 16384 rows; at 7 and 8 bits up to 192 on at most 8192 rows
+    assert fused_gemm_pays(256, 11008, 4, 4096) and fused_gemm_pays(256, 28672, 5, 8192) and fused_gemm_pays(256, 13824, 6, 5120)
+    assert not fused_gemm_pays(129, 28672, 6, 8192) and fused_gemm_pays(192, 8192, 8, 8192) and not fused_gemm_pays(193, 8192, 8, 8192)
+    assert not fused_gemm_pays(129, 11008, 8, 4096) and fused_gemm_pays(256, 4096, 8, 4096) and not fused_gemm_pays(256, 4096, 8, 11008)
+    # up to 512 at 3 bits on at most 8192 rows
+    assert fused_gemm_pays(512, 4096, 3, 11008) and fused_gemm_pays(512, 8192, 3, 8192) and not fused_gemm_pays(257, 11008, 3, 4096)
+    assert not fused_gemm_pays(513, 4096, 3, 4096) and not fused_gemm_pays(257, 4096, 4, 4096)
+    # linears of 1024..4095 rows: 3 and 4 bits up to 512
+    assert fused_gemm_pays(100, 1024, 3, 4096) and fused_gemm_pays(512, 1024, 4, 8192) and not fused_gemm_pays(100, 1024, 5, 4096)
+    assert not fused_gemm_pays(100, 512, 3, 4096)

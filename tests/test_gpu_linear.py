@@ -115,15 +115,16 @@ def test_forward_group_equals_module_by_module(oracle):
 
 
 def test_forward_takes_the_tiled_gemm_up_to_256_rows_at_3_and_4_bits(oracle):
-    """A linear of 4096 rows of a multiple of 128 elements: 3 bits go through the fused GEMM up to 256 activation rows,
-    4 and 5 bits too on rows this short (3 bits up to 512 on a linear of 4096 rows), 6 bits and 513 rows through dequant + matmul; all
-    against the oracle."""
+    """A linear of 4096 rows of a multiple of 128 elements: up to 6 bits go through the fused GEMM up to 256 activation
+    rows (3 bits up to 512), 6 bits beyond 256 rows and anything beyond 512 through dequant + matmul; all against the
+    oracle."""
     from any_precision_amd.linear import fused_gemm_pays
     L = make(4096, 256, seed=5)
     m, _ = _module(L, bias=False)
     assert fused_gemm_pays(200, 4096, 3, 256) and fused_gemm_pays(256, 4096, 4, 256)
-    assert fused_gemm_pays(200, 4096, 5, 256) and not fused_gemm_pays(200, 4096, 6, 256) and fused_gemm_pays(257, 4096, 3, 256) and not fused_gemm_pays(513, 4096, 3, 256)
-    for b, M in ((3, 200), (3, 256), (4, 256), (5, 200), (6, 200), (3, 257), (3, 513)):
+    assert fused_gemm_pays(200, 4096, 5, 256) and fused_gemm_pays(200, 4096, 6, 256) and not fused_gemm_pays(257, 4096, 6, 256)
+    assert fused_gemm_pays(257, 4096, 3, 256) and not fused_gemm_pays(513, 4096, 3, 256)
+    for b, M in ((3, 200), (3, 256), (4, 256), (5, 200), (6, 200), (6, 257), (8, 256), (3, 257), (3, 513)):
         print(f"linear tiled b={b} M={M}", flush=True)
         x = synth.make_x(M, L.K, seed=M)
         y = m(torch.from_numpy(x).cuda(), precision=b)
@@ -136,7 +137,8 @@ def test_forward_group_beyond_32_rows_is_one_tiled_launch(oracle):
     says so, with biases added afterwards; against the oracle, joined or as a list."""
     from any_precision_amd.linear import forward_group, fused_set_pays
     assert fused_set_pays(128, [4096, 4096, 4096], 3, 4096) and fused_set_pays(256, [11008, 11008], 5, 4096)
-    assert fused_set_pays(64, [11008, 11008], 8, 4096) and not fused_set_pays(128, [11008, 11008], 8, 4096)
+    assert fused_set_pays(128, [11008, 11008], 8, 4096) and not fused_set_pays(129, [11008, 11008], 8, 4096)
+    assert fused_set_pays(256, [4096, 4096, 4096], 8, 4096)
     assert fused_set_pays(128, [4096, 1024, 1024], 8, 4096) and fused_set_pays(9, [4096, 4096], 3, 4096)
     assert not fused_set_pays(32, [11008, 11008], 3, 4096) and not fused_set_pays(8, [4096, 4096], 3, 4096)
     assert fused_set_pays(16, [8192, 1024, 1024], 8, 8192) and not fused_set_pays(16, [8192, 8200], 8, 8192)
