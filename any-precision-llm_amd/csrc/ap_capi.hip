@@ -423,7 +423,7 @@ bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *
     geo->kh = mbw < 4 || (mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && small <= cu_count()))) ? 2 : 1;
     geo->grid_n = (int)tiles_n;  // tiles of 64 weight rows (of all linears of the launch)
     geo->grid_m = (M + 16 * mbw - 1) / (16 * mbw);
-    return geo->grid_m <= 65535;
+    return (tiles_n + 7) / 8 * 8 * (long long)geo->grid_m <= 0x7fffffffLL;  // a one-dimensional grid, padded to groups of 8
 }
 
 // Where the tiled kernel is the fastest fused form (same sweep, and the linear shapes of the 7B / 8B / 13B / 70B layers

@@ -91,20 +91,28 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     const int tid = wv * kWave + lane;                            // thread within the half
     const int col = lane & 15, grp = lane >> 4;
     const int W = K >> 5;
+    // Workgroup -> tile.  Consecutive workgroups go round-robin to the 8 XCDs, each with its own L2, and the tiles of
+    // one block of weight rows over the activation rows read the same planes: they get workgroup numbers 8 apart, so
+    // that they run on one XCD at about the same time and the planes come from HBM once.  Workgroup id = 8 (grid_m a +
+    // m) + c stands for weight-row tile 8 a + c and activation-row tile m (the grid is padded to whole groups of 8).
+    const int grid_m = (M + BM - 1) / BM;
+    const int wg = blockIdx.x, wa = wg / (8 * grid_m), wr = wg % (8 * grid_m);
+    const int tile_n = 8 * wa + (wr & 7), tile_m = wr >> 3;
+    if (tile_n >= mem.tile0[mem.count]) return;  // padding (workgroup-uniform)
     // the linear this tile belongs to (workgroup-uniform) and the tile's place in it
     int g = 0;
 #pragma unroll
     for (int i = 1; i < kGemmtMaxGroup; i++)
-        if (i < mem.count && (int)blockIdx.x >= mem.tile0[i]) g = i;
+        if (i < mem.count && tile_n >= mem.tile0[i]) g = i;
     const uint32_t *__restrict__ qweight = mem.qweight[g];
     const half_t *__restrict__ lut = reinterpret_cast<const half_t *>(mem.lut[g]);
     half_t *__restrict__ out = reinterpret_cast<half_t *>(mem.out[g]);
     const int N = mem.N[g];
     const long long ldo = mem.ldo[g];
-    const int nb = ((int)blockIdx.x - mem.tile0[g]) * BN;  // first weight row of the workgroup
+    const int nb = (tile_n - mem.tile0[g]) * BN;  // first weight row of the workgroup
     const size_t plane_stride = (size_t)N * W;
     const int n0 = nb + wv * WROWS;     // ... of this wave
-    const int m0 = blockIdx.y * BM;     // first activation row of the tile
+    const int m0 = tile_m * BM;         // first activation row of the tile
     const int steps = (W + 15) >> 4;    // 16 words of every row per step
     const int nit = (steps + KH - 1) / KH;   // steps per K half; a half with one step fewer idles through the last
     // (all workgroups walk K in the same order: those in flight then read the same columns of the activations at

@@ -11,7 +11,8 @@ namespace ap {
 template <int BITS>
 void launch_gemmt(const GemmtGeometry &geo, const uint16_t *x, const GemmtMembers &members, int M, int K, hipStream_t stream) {
     const half_t *xh = reinterpret_cast<const half_t *>(x);
-    const dim3 block(kWave, kGemmtWaves * geo.kh), grid(geo.grid_n, geo.grid_m);
+    // one-dimensional grid, weight-row tiles padded to groups of 8 (the kernel maps a workgroup to its tile)
+    const dim3 block(kWave, kGemmtWaves * geo.kh), grid((unsigned)((geo.grid_n + 7) / 8 * 8) * (unsigned)geo.grid_m);
     // one block of 16 weight rows per wave: two measured slower on every shape (a quarter of the workgroups, and the
     // LDS traffic per matrix instruction falls by less than a third)
     if (geo.mbw == 8)
