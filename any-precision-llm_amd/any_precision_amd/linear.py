@@ -66,9 +66,12 @@ def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bo
     members (gate/up) at 9..32 rows are as fast module by module -- up to 128 rows at every bit-width (q/k/v of the 7B layer at 128 rows, 3 bits: 33 us against 44 one by one and
     128 for three dequant + GEMM pairs; gate/up at 8 bits: 96 against 115 for the pairs), up to 256 at up to 6 bits
     (gate/up at 5 bits: 105 against 145) and, at 7 and 8 bits, where every member has fewer than 8192 rows (q/k/v at 8
-    bits: 94 against 114; gate/up: 145 against 149)."""
-    if in_features % 128 or not 8 < rows <= 256 or sum(out_features) < 4096:
+    bits: 94 against 114; gate/up: 145 against 149); up to 512 at 3 bits where no member has more than 8192 rows, as
+    each member alone would."""
+    if in_features % 128 or not 8 < rows <= 512 or sum(out_features) < 4096:
         return False
+    if rows > 256:      # where every member alone would take the fused GEMM (fused_gemm_pays): 3 bits, up to 8192 rows
+        return w_bits == 3 and max(out_features) <= 8192
     if rows <= 32:
         return max(out_features) <= 8192 and in_features >= 1024
     return rows <= 128 or w_bits <= 6 or max(out_features) < 8192

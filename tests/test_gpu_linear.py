@@ -142,11 +142,13 @@ def test_forward_group_beyond_32_rows_is_one_tiled_launch(oracle):
     assert fused_set_pays(128, [4096, 1024, 1024], 8, 4096) and fused_set_pays(9, [4096, 4096], 3, 4096)
     assert not fused_set_pays(32, [11008, 11008], 3, 4096) and not fused_set_pays(8, [4096, 4096], 3, 4096)
     assert fused_set_pays(16, [8192, 1024, 1024], 8, 8192) and not fused_set_pays(16, [8192, 8200], 8, 8192)
-    assert not fused_set_pays(257, [4096, 4096], 3, 4096) and not fused_set_pays(64, [4096, 4096], 3, 4000)
+    assert fused_set_pays(257, [4096, 4096], 3, 4096) and not fused_set_pays(257, [4096, 4096], 4, 4096)
+    assert not fused_set_pays(513, [4096, 4096], 3, 4096) and not fused_set_pays(300, [11008, 11008], 3, 4096)
+    assert not fused_set_pays(64, [4096, 4096], 3, 4000)
     layers = [make(n, 256, seed=80 + n) for n in (4096, 512, 520)]
     for bias in (False, True):
         mods = [_module(L, bias=bias)[0] for L in layers]
-        for b, rows in ((3, 40), (8, 64), (5, 200), (8, 200)):
+        for b, rows in ((3, 40), (8, 64), (5, 200), (8, 200), (3, 300)):
             print(f"forward_group tiled bias={bias} b={b} rows={rows}", flush=True)
             x = synth.make_x(rows, 256, seed=rows)
             xg = torch.from_numpy(x).cuda()
