@@ -65,10 +65,11 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     //           table as below;
     //   4..8 bits: the plain table with one fp16 entry per dword; two copies up to 7 bits in the two-half form
     //           (16..64 KB per workgroup), one copy at 8 bits (64 KB) and with one group of waves (up to 6 bits there:
-    //           1..16 KB; the tables of 7 and 8 bits would cost a workgroup per CU).
+    //           1..16 KB; the tables of 7 and 8 bits would cost a workgroup per CU -- except the 128-row tile at 8
+    //           bits, which has its CU to itself already).
     constexpr bool CF = BITS == 3 && RB == 1;
     constexpr bool CF4 = BITS == 4 && RB == 1 && KH == 2;
-    constexpr bool CF16 = !PAIR && RB == 1 && (KH == 2 || BITS <= 6);
+    constexpr bool CF16 = !PAIR && RB == 1 && (KH == 2 || BITS <= 6 || (BITS == 8 && MBW == 8));
     constexpr int SLOTS = (KH == 1 || BITS == 8) ? 16 : 32;
     constexpr int ESHIFT = SLOTS == 32 ? 7 : 6;  // log2 of the bytes of an entry
     __shared__ uint32_t cftab[CF ? kGemmtWaves * 64 * SLOTS : (CF4 ? kGemmtWaves * 256 * 16 : (CF16 ? kGemmtWaves * NC * SLOTS : 1))];
