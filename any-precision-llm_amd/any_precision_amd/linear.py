@@ -28,8 +28,8 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
     * rows of a multiple of 128 elements (the tiled kernel), linears of at least 4096 rows: up to 128 activation rows
       at every bit-width (11008 x 4096, 8 bits: 50 / 58; 28672 x 8192: 189 / 234; 5120 x 13824: 93 / 113); up to 256
       at up to 5 bits (11008 x 4096, 4 bits: 58 / 73; 13824 x 5120, 5 bits: 79 / 97), at 6 bits except on linears of
-      more than 16384 rows (28672 x 8192: 263 / 250), at 7 and 8 bits up to 192 on linears of at most 8192 rows
-      (8192 x 8192, 8 bits: 89 / 103; 11008 x 4096: 96 / 66) and up to 256 on 4096 x 4096 (33 / 39); up to 512 at
+      more than 16384 rows (28672 x 8192: 263 / 250), at 7 and 8 bits on linears of at most 8192 rows
+      (8192 x 8192, 8 bits: 87 / 116; 5120 x 5120: 56 / 69; 4096 x 11008: 82 / 82; 11008 x 4096: 96 / 66); up to 512 at
       3 bits on linears of at most 8192 rows (4096 x 11008: 87 / 99; 8192 x 8192: 101 / 114; 14336 x 4096: 99 / 90);
     * the same rows on linears of 1024..4095 rows: up to 512 activation rows at 3 and 4 bits (1024 x 4096: 11-15 /
       18-23; at 6 bits and more the pair wins);
@@ -47,7 +47,7 @@ def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int 
             if rows <= 256:
                 if w_bits <= 6:
                     return w_bits <= 5 or out_features <= 16384
-                return (rows <= 192 and out_features <= 8192) or (out_features <= 4096 and in_features <= 4096)
+                return out_features <= 8192
             return w_bits == 3 and out_features <= 8192
         if out_features >= 1024 and w_bits <= 4:
             return True

@@ -409,7 +409,13 @@ bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *
         if (forced < 4 && K < 1024) return false;  // tiles of 16 and 32 rows exist in the two-half form only
         mbw = forced;
     } else if (M > 64) {
-        if (10 * small >= (w_bits == 3 ? 30LL : 13LL) * cu_count()) mbw = 8;
+        // Tiles of 128 activation rows once the 64-row tiles no longer fit the CUs in one round of the two-half form --
+        // from 5 bits on as soon as they exceed the CUs (5120 x 5120 at 256 rows, 320 tiles: 47 / 49 / 56 us at 5 / 6 / 8
+        // bits against 52 / 56 / 73 with one group of waves per 64-row tile); at 4 bits, whose two-half form has the
+        // pair table, from 1.5 tiles per CU (up to there two rounds of that form: 44 us against 47); at 3 bits from 3
+        // tiles per CU (one group of waves per 64-row tile is as fast up to there).
+        const long long cus = cu_count();
+        if (w_bits == 3 ? small >= 3 * cus : (w_bits == 4 ? 2 * small > 3 * cus : small > cus)) mbw = 8;
     }
     // A grid that leaves CUs idle takes the narrowest tile that still gives no CU a second workgroup: more workgroups
     // dequantise the same weights, each for fewer activation rows (4096 x 4096 at 64 rows, 3 bits: 14 us with four
@@ -420,7 +426,8 @@ bool gemmt_geometry(int M, long long tiles_n, int K, int w_bits, GemmtGeometry *
     }
     geo->mbw = mbw;
     // two K halves need at least two steps of 512 elements
-    geo->kh = mbw < 4 || (mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && small <= cu_count()))) ? 2 : 1;
+    const bool halves = small <= cu_count() || (w_bits == 4 && 2 * small <= 3 * (long long)cu_count());
+    geo->kh = mbw < 4 || (mbw == 4 && K >= 1024 && (force_kh == 2 || (force_kh <= 0 && halves))) ? 2 : 1;
     geo->grid_n = (int)tiles_n;  // tiles of 64 weight rows (of all linears of the launch)
     geo->grid_m = (M + 16 * mbw - 1) / (16 * mbw);
     return (tiles_n + 7) / 8 * 8 * (long long)geo->grid_m <= 0x7fffffffLL;  // a one-dimensional grid, padded to groups of 8

@@ -61,10 +61,10 @@ def test_fused_gemm_dispatch_rule():
     # the tiled kernel, linears of at least 4096 rows: every bit-width up to 128 activation rows
     assert all(fused_gemm_pays(128, n, b, k) for b in (3, 8) for n, k in ((4096, 4096), (11008, 4096), (5120, 13824), (28672, 8192)))
     assert fused_gemm_pays(65, 14336, 8, 4096) and fused_gemm_pays(64, 5120, 8, 13824) and fused_gemm_pays(64, 8192, 8, 8192)
-    # up to 256 at up to 5 bits; at 6 bits except beyond 16384 rows; at 7 and 8 bits up to 192 on at most 8192 rows
+    # up to 256 at up to 5 bits; at 6 bits except beyond 16384 rows; at 7 and 8 bits on at most 8192 rows
     assert fused_gemm_pays(256, 11008, 4, 4096) and fused_gemm_pays(256, 28672, 5, 8192) and fused_gemm_pays(256, 13824, 6, 5120)
-    assert not fused_gemm_pays(129, 28672, 6, 8192) and fused_gemm_pays(192, 8192, 8, 8192) and not fused_gemm_pays(193, 8192, 8, 8192)
-    assert not fused_gemm_pays(129, 11008, 8, 4096) and fused_gemm_pays(256, 4096, 8, 4096) and not fused_gemm_pays(256, 4096, 8, 11008)
+    assert not fused_gemm_pays(129, 28672, 6, 8192) and fused_gemm_pays(256, 8192, 8, 8192) and not fused_gemm_pays(257, 8192, 8, 8192)
+    assert not fused_gemm_pays(129, 11008, 8, 4096) and fused_gemm_pays(256, 4096, 8, 4096) and fused_gemm_pays(256, 5120, 7, 13824)
     # up to 512 at 3 bits on at most 8192 rows
     assert fused_gemm_pays(512, 4096, 3, 11008) and fused_gemm_pays(512, 8192, 3, 8192) and not fused_gemm_pays(257, 11008, 3, 4096)
     assert not fused_gemm_pays(513, 4096, 3, 4096) and not fused_gemm_pays(257, 4096, 4, 4096)
