@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_PKG_ROOT, "lib", "libanyprec_hip.so")
 
 AP_OK = 0
 AP_ENULL, AP_EBITS, AP_ESHAPE, AP_EALIGN, AP_EBATCH, AP_ELIMIT, AP_EKNOB = -1, -2, -3, -4, -5, -6, -7
-AP_ABI_VERSION = 7
+AP_ABI_VERSION = 8
 
 if not os.path.exists(LIB_PATH):
     raise ModuleNotFoundError(
@@ -35,6 +35,12 @@ lib.ap_gemm_kbit.argtypes = [_vp, _vp, _vp, _vp, _ci, _ci, _ci, _ci, _vp]
 lib.ap_gemm_kbit.restype = _ci
 _pi = ctypes.POINTER(ctypes.c_int)
 _pvp = ctypes.POINTER(ctypes.c_void_p)
+lib.ap_dequant_kbit_group.argtypes = [_ci, _pvp, _pvp, _pvp, _pi, _pi, _ci, _vp]
+lib.ap_dequant_kbit_group.restype = _ci
+lib.ap_gemm_kbit_pays.argtypes = [_ci, _ci, _ci, _ci]
+lib.ap_gemm_kbit_pays.restype = _ci
+lib.ap_gemm_kbit_group_pays.argtypes = [_ci, _pi, _ci, _ci, _ci]
+lib.ap_gemm_kbit_group_pays.restype = _ci
 lib.ap_matmul_kbit_group.argtypes = [_vp, _ci, _pvp, _pvp, _pvp, _pi, _ci, _ci, _ci, _vp]
 lib.ap_matmul_kbit_group.restype = _ci
 _pll = ctypes.POINTER(ctypes.c_longlong)
@@ -74,9 +80,38 @@ if lib.ap_abi_version() != AP_ABI_VERSION:
 
 EXPORTS = ("ap_abi_version", "ap_strerror", "ap_dequant_kbit", "ap_matmul_kbit", "ap_matmul_kbit_group",
            "ap_gemm_kbit", "ap_matmul_kbit_geometry", "ap_set_tuning", "ap_get_tuning", "ap_probe_stream", "ap_probe_empty", "ap_probe_write", "ap_matmul_kbit_route", "ap_matmul_kbit_group_route",
-           "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu", "ap_decode_advance", "ap_gemm_kbit_group")
+           "ap_add_rmsnorm", "ap_silu_mul", "ap_decode_attention", "ap_matmul_kbit_swiglu", "ap_decode_advance", "ap_gemm_kbit_group", "ap_dequant_kbit_group", "ap_gemm_kbit_pays",
+           "ap_gemm_kbit_group_pays")
 GEMM_MAX_M = 128
 GROUP_MAX = 4
+DEQUANT_GROUP_MAX = 8
+
+
+def dequant_group(qweights, luts, outs, rows, cols, w_bits: int, stream: int) -> int:
+    """ap_dequant_kbit_group on raw device addresses (lists of equal length <= DEQUANT_GROUP_MAX)."""
+    n = len(qweights)
+    arr = ctypes.c_void_p * n
+    ints = ctypes.c_int * n
+    return lib.ap_dequant_kbit_group(n, arr(*qweights), arr(*luts), arr(*outs), ints(*rows), ints(*cols), w_bits, stream)
+
+
+def gemm_pays(M: int, N: int, K: int, w_bits: int) -> bool:
+    """ap_gemm_kbit_pays: the fused GEMM beats dequant_kbit + a library GEMM for this shape."""
+    rc = lib.ap_gemm_kbit_pays(M, N, K, w_bits)
+    if rc < 0:
+        check(rc, "ap_gemm_kbit_pays")
+    return rc == 1
+
+
+def gemm_group_pays(M: int, rows, K: int, w_bits: int) -> bool:
+    """ap_gemm_kbit_group_pays: one tiled launch over the set beats its members one by one."""
+    n = len(rows)
+    if not 1 <= n <= GROUP_MAX:
+        return False
+    rc = lib.ap_gemm_kbit_group_pays(n, (ctypes.c_int * n)(*rows), M, K, w_bits)
+    if rc < 0:
+        check(rc, "ap_gemm_kbit_group_pays")
+    return rc == 1
 
 
 def matmul_group(x_ptr: int, qweights, luts, outs, rows, M: int, K: int, w_bits: int, stream: int) -> int:
@@ -115,7 +150,7 @@ def matmul_geometry(M: int, N: int, K: int, w_bits: int) -> dict:
     return dict(zip(("wpl", "segments", "rows", "grid"), (v.value for v in vals)))
 
 
-ROUTES = ("dot", "stream", "fine", "persist", "mfma4", "mfma16")
+ROUTES = ("dot", "stream", "fine", "mfma4", "mfma16")
 
 
 def matmul_route(M: int, N: int, K: int, w_bits: int) -> str:

@@ -5,8 +5,8 @@ Same constructor, buffers (``qweight`` int32 ``[max(supported_bits), out, in/32]
 ``lut{b}`` fp16 ``[out, 2**b]``, optional ``bias`` buffer), state-dict keys,
 ``forward(x, precision=...)``, ``set_precision`` and ``prune_precisions``.
 Batch dispatch: up to 8 activation rows -> ``matmul_kbit`` as in the reference (:60-64);
-9 .. 32 rows (.. 64, 128 or 256 where ``fused_gemm_pays`` says so) -> the fused ``gemm_kbit``; beyond ->
-``dequant_kbit`` + ``torch.matmul`` as in the reference.
+9 .. 32 rows (up to 64, 128, 256 or 512 where the library's ``ap_gemm_kbit_pays`` says so) -> the fused
+``gemm_kbit``; beyond -> ``dequant_kbit`` + ``torch.matmul`` as in the reference.
 """
 from __future__ import annotations
 
@@ -16,65 +16,22 @@ import torch.nn as nn
 try:
     from any_precision_ext import (matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, gemm_kbit_group,
                                    GEMM_MAX_M)
+    from . import _capi
 except ModuleNotFoundError:
     matmul_kbit, matmul_kbit_group, matmul_kbit_swiglu, dequant_kbit, gemm_kbit, gemm_kbit_group, GEMM_MAX_M = (None,) * 6 + (0,)
+    _capi = None
 
 
-def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int = 0) -> bool:
-    """Whether the fused GEMM beats dequant_kbit + torch.matmul.  Measured on the linear shapes of the Llama-2-7B /
-    Llama-3-8B / 13B / 70B layers at 96..512 activation rows and every bit-width (fused / pair, us):
-
-    * always up to 32 activation rows (1.3-4x at 16);
-    * rows of a multiple of 128 elements (the tiled kernel), linears of at least 4096 rows: up to 128 activation rows
-      at every bit-width (11008 x 4096, 8 bits: 50 / 58; 28672 x 8192: 189 / 234; 5120 x 13824: 93 / 113); up to 256
-      at up to 5 bits (11008 x 4096, 4 bits: 58 / 73; 13824 x 5120, 5 bits: 79 / 97), at 6 bits except on linears of
-      more than 16384 rows (28672 x 8192: 263 / 250), at 7 and 8 bits on linears of at most 8192 rows
-      (8192 x 8192, 8 bits: 87 / 116; 5120 x 5120: 56 / 69; 4096 x 11008: 82 / 82; 11008 x 4096: 96 / 66); up to 512 at
-      3 bits on linears of at most 8192 rows (4096 x 11008: 87 / 99; 8192 x 8192: 101 / 114; 14336 x 4096: 99 / 90);
-    * the same rows on linears of 1024..4095 rows: up to 512 activation rows at 3 and 4 bits (1024 x 4096: 11-15 /
-      18-23; at 6 bits and more the pair wins);
-    * other row lengths (the K-split kernel only): up to 64 on linears of fewer than 8192 rows, and on larger ones at up
-      to 5 bits -- except, on rows of more than 4096 elements, from 6 bits on linears of 5120 rows or more and from 5
-      bits on linears of at most 2048 rows; up to 128 on linears of 4096..8191 rows of at most 4096 elements.
-
-    Beyond, one table lookup per weight and tile of activation rows costs more than materialising the weight once."""
-    if rows <= min(32, GEMM_MAX_M):
-        return True
-    if GEMM_MAX_M and in_features > 0 and in_features % 128 == 0 and rows <= 512:
-        if out_features >= 4096:
-            if rows <= 128:
-                return True
-            if rows <= 256:
-                if w_bits <= 6:
-                    return w_bits <= 5 or out_features <= 16384
-                return out_features <= 8192
-            return w_bits == 3 and out_features <= 8192
-        if out_features >= 1024 and w_bits <= 4:
-            return True
-    if rows <= min(64, GEMM_MAX_M):
-        if in_features > 4096 and ((w_bits >= 6 and out_features >= 5120) or (w_bits >= 5 and out_features <= 2048)):
-            return False
-        return out_features < 8192 or w_bits <= 5
-    return rows <= min(128, GEMM_MAX_M) and 4096 <= out_features < 8192 and 0 < in_features <= 4096
+def fused_gemm_pays(rows: int, out_features: int, w_bits: int, in_features: int) -> bool:
+    """Whether the fused GEMM beats ``dequant_kbit`` + ``torch.matmul`` for ``rows`` activation rows: the library's own
+    measured crossovers (``ap_gemm_kbit_pays``; the thresholds live in one place, beside the kernels' launch rules)."""
+    return _capi.gemm_pays(rows, out_features, in_features, w_bits)
 
 
 def fused_set_pays(rows: int, out_features, w_bits: int, in_features: int) -> bool:
     """Whether ONE launch of the tiled GEMM over linears that share their input (``gemm_kbit_group``) beats calling them
-    one by one, each through whatever ``fused_gemm_pays`` picks (measured on the q/k/v and gate/up sets of the
-    Llama-2-7B / Llama-3-8B / 13B layers at 16..256 rows): from 33 rows on -- from 9 where every member has at most
-    8192 rows (q/k/v of the 7B layer at 16 rows, 3 bits: 16 us against 23; of the 13B layer: 20 against 36); wide
-    members (gate/up) at 9..32 rows are as fast module by module -- up to 128 rows at every bit-width (q/k/v of the 7B layer at 128 rows, 3 bits: 33 us against 44 one by one and
-    128 for three dequant + GEMM pairs; gate/up at 8 bits: 96 against 115 for the pairs), up to 256 at up to 6 bits
-    (gate/up at 5 bits: 105 against 145) and, at 7 and 8 bits, where every member has fewer than 8192 rows (q/k/v at 8
-    bits: 94 against 114; gate/up: 145 against 149); up to 512 at 3 bits where no member has more than 8192 rows, as
-    each member alone would."""
-    if in_features % 128 or not 8 < rows <= 512 or sum(out_features) < 4096:
-        return False
-    if rows > 256:      # where every member alone would take the fused GEMM (fused_gemm_pays): 3 bits, up to 8192 rows
-        return w_bits == 3 and max(out_features) <= 8192
-    if rows <= 32:
-        return max(out_features) <= 8192 and in_features >= 1024
-    return rows <= 128 or w_bits <= 6 or max(out_features) < 8192
+    one by one (``ap_gemm_kbit_group_pays``)."""
+    return _capi.gemm_group_pays(rows, list(out_features), in_features, w_bits)
 
 
 def forward_group(modules, x, precision=None, concat=False):

@@ -22,7 +22,7 @@ import torch
 
 from any_precision_amd import _capi
 
-__all__ = ["matmul_kbit", "dequant_kbit", "gemm_kbit", "gemm_kbit_group", "matmul_kbit_group", "matmul_kbit_swiglu", "GEMM_MAX_M"]
+__all__ = ["matmul_kbit", "dequant_kbit", "dequant_kbit_group", "gemm_kbit", "gemm_kbit_group", "matmul_kbit_group", "matmul_kbit_swiglu", "GEMM_MAX_M"]
 
 GEMM_MAX_M = _capi.GEMM_MAX_M
 
@@ -62,6 +62,24 @@ def dequant_kbit(qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch
                                   torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "dequant_kbit")
     return out
+
+
+def dequant_kbit_group(qweights, luts, w_bits: int):
+    """``[dequant_kbit(q, t, w_bits) for q, t in zip(qweights, luts)]`` in ONE launch: up to DEQUANT_GROUP_MAX linears of
+    any shapes on one GPU at one bit-width (a decoder layer has seven).  No counterpart in the reference, which launches
+    its kernel once per linear (main.cu:82-84); results are bit-identical to the separate calls."""
+    if len(qweights) != len(luts) or not 1 <= len(qweights) <= _capi.DEQUANT_GROUP_MAX:
+        raise ValueError(f"dequant_kbit_group: need 1..{_capi.DEQUANT_GROUP_MAX} (qweight, lut) pairs")
+    shapes = [_check_weight(q, t, w_bits, "dequant_kbit_group") for q, t in zip(qweights, luts)]
+    dev = qweights[0].device
+    if any(q.device != dev for q in qweights):
+        raise ValueError("dequant_kbit_group: all weights must be on one device")
+    with torch.cuda.device(dev):
+        outs = [torch.empty((N, K), dtype=torch.float16, device=dev) for N, K in shapes]
+        rc = _capi.dequant_group([q.data_ptr() for q in qweights], [t.data_ptr() for t in luts], [o.data_ptr() for o in outs],
+                                 [N for N, _ in shapes], [K for _, K in shapes], w_bits, torch.cuda.current_stream().cuda_stream)
+    _capi.check(rc, "dequant_kbit_group")
+    return outs
 
 
 def matmul_kbit(in_: torch.Tensor, qweight: torch.Tensor, lut: torch.Tensor, w_bits: int) -> torch.Tensor:
@@ -159,6 +177,12 @@ def gemm_kbit_group(in_: torch.Tensor, qweights, luts, w_bits: int, concat: bool
             outs = [torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device) for N in rows]
         rc = _capi.gemm_group(in_.data_ptr(), [q.data_ptr() for q in qweights], [t.data_ptr() for t in luts],
                               [o.data_ptr() for o in outs], rows, ldo, M, K, w_bits, torch.cuda.current_stream().cuda_stream)
+        if rc == _capi.AP_ELIMIT and joint is not None:
+            # beyond the tiled kernel's geometry (it alone writes side by side): dense results, joined below
+            joint = None
+            outs = [torch.empty(in_.shape[:-1] + (N,), dtype=torch.float16, device=in_.device) for N in rows]
+            rc = _capi.gemm_group(in_.data_ptr(), [q.data_ptr() for q in qweights], [t.data_ptr() for t in luts],
+                                  [o.data_ptr() for o in outs], rows, None, M, K, w_bits, torch.cuda.current_stream().cuda_stream)
     _capi.check(rc, "gemm_kbit_group")
     if concat:
         return joint if joint is not None else torch.cat(outs, dim=-1)

@@ -58,7 +58,6 @@ def build_hip(verbose: bool = False, extra_flags=(), jobs: int = 8) -> str:
     for b in range(3, 9):
         units.append((os.path.join(CSRC, "ap_gemv_inst.hip"), os.path.join(OBJDIR, f"ap_gemv_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemvf_inst.hip"), os.path.join(OBJDIR, f"ap_gemvf_b{b}.o"), [f"-DAP_BITS={b}"]))
-        units.append((os.path.join(CSRC, "ap_gemvr_inst.hip"), os.path.join(OBJDIR, f"ap_gemvr_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemvp_inst.hip"), os.path.join(OBJDIR, f"ap_gemvp_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemm_inst.hip"), os.path.join(OBJDIR, f"ap_gemm_b{b}.o"), [f"-DAP_BITS={b}"]))
         units.append((os.path.join(CSRC, "ap_gemmw_inst.hip"), os.path.join(OBJDIR, f"ap_gemmw_b{b}.o"), [f"-DAP_BITS={b}"]))

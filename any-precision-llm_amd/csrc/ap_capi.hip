@@ -13,7 +13,6 @@
 #include "ap_gemv_launch.hpp"
 #include "ap_gemvf_launch.hpp"
 #include "ap_gemvp_launch.hpp"
-#include "ap_gemvr_launch.hpp"
 #include "ap_probe.hpp"
 
 namespace {
@@ -40,8 +39,6 @@ enum {
     kGemvStream,        // row-streaming GEMV: 0 never, 1 where it pays, 2 wherever it fits
     kGemvStreamWaves,   // waves per CU the row-streaming GEMV grid aims for
     kGemvFine,          // fine-grained row-pair GEMV: 0 never, 1 where it pays, 2 wherever it fits
-    kGemvPersist,       // persistent row-loop GEMV: 0 never, 1 where it pays, 2 wherever it fits
-    kGemvPersistWaves,  // waves per CU the persistent GEMV grid aims for
     kGemmWalk,          // row-walking fused GEMM: 0 never, 1 where it pays, 2 wherever it fits
     kGemmWalkWgs,       // workgroups per CU its grid aims for
     kGemmTiled,         // tiled fused GEMM (ap_gemm_kbit): 0 never, 1 where it pays, 2 wherever it fits
@@ -53,7 +50,7 @@ Knob g_knobs[kKnobCount] = {
     {"gemv_target_waves", 16384}, {"gemv_rows", 0},      {"gemv_wpl", 0},     {"dequant_blocks_per_cu", 0},
     {"matmul_mfma_from", 5},      {"gemm_split", 0},     {"matmul_mfma4", 1}, {"gemv4_groups", 0},
     {"gemm_rb2", 1},              {"gemv_stream", 1},    {"gemv_stream_waves", 24},
-    {"gemv_fine", 1},             {"gemv_persist", 1},   {"gemv_persist_waves", 8},
+    {"gemv_fine", 1},
     {"gemm_walk", 1},             {"gemm_walk_wgs", 1},  {"gemm_tiled", 1},   {"gemm_tile", 0},
     {"gemm_tile_split", 0},
 };
@@ -171,18 +168,18 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     return AP_OK;
 }
 
+// One launch of the dequantiser over `count` linears (arguments already checked): fills the member table and sizes the grid.
 template <int BITS>
-void launch_dequant(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, hipStream_t stream) {
-    const int S = ((K >> 5) + kWave - 1) / kWave;  // 64-word segments per row
-    long long blocks = ((long long)N * S + kDequantWaves - 1) / kDequantWaves;
+void launch_dequant(const DequantMembers &mem, long long weights, hipStream_t stream) {
+    const long long items = mem.item_end[mem.count - 1];  // 64-word segments of all members
+    long long blocks = (items + kDequantWaves - 1) / kDequantWaves;
     // Workgroups per CU the grid is capped at (the kernel strides over the rest): 32 measured best or within 1 % of
     // best on every 7B..70B shape against 2..64; from about 128 M weights 64 is 5-6 % faster (28672 x 8192: a shorter
     // tail).  The knob overrides when positive.
-    const int per_cu = knob(kDequantBlocksPerCu) > 0 ? knob(kDequantBlocksPerCu) : ((long long)N * K >= (128LL << 20) ? 64 : 32);
+    const int per_cu = knob(kDequantBlocksPerCu) > 0 ? knob(kDequantBlocksPerCu) : (weights >= (128LL << 20) ? 64 : 32);
     const long long cap = (long long)cu_count() * per_cu;
     if (blocks > cap) blocks = cap;
-    dequant_kbit_kernel<BITS><<<dim3((unsigned)blocks), dim3(kDequantWaves * kWave), 0, stream>>>(
-        qweight, reinterpret_cast<const half_t *>(lut), reinterpret_cast<half_t *>(out), N, K);
+    dequant_kbit_kernel<BITS><<<dim3((unsigned)blocks), dim3(kDequantWaves * kWave), 0, stream>>>(mem);
 }
 
 // hipGetLastError() returns AND clears the thread's sticky error, whoever left it: an entry point
@@ -335,19 +332,41 @@ int ap_decode_attention(const uint16_t *qkv, const float *cos_table, const float
 
 int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int N, int K, int w_bits,
                     void *stream) {
-    if (!qweight || !lut || !out) return AP_ENULL;
-    const int rc = check_common(N, K, w_bits);
-    if (rc != AP_OK) return rc;
-    if (!aligned16(qweight) || !aligned16(lut) || !aligned16(out)) return AP_EALIGN;
+    return ap_dequant_kbit_group(1, &qweight, &lut, &out, &N, &K, w_bits, stream);
+}
+
+int ap_dequant_kbit_group(int count, const uint32_t *const *qweight, const uint16_t *const *lut, uint16_t *const *out,
+                          const int *N, const int *K, int w_bits, void *stream) {
+    if (!qweight || !lut || !out || !N || !K) return AP_ENULL;
+    if (count < 1 || count > kDequantMaxGroup) return AP_ELIMIT;
+    DequantMembers mem = {};
+    long long items = 0, weights = 0;
+    for (int g = 0; g < count; g++) {
+        if (!qweight[g] || !lut[g] || !out[g]) return AP_ENULL;
+        const int rc = check_common(N[g], K[g], w_bits);
+        if (rc != AP_OK) return rc;
+        if (!aligned16(qweight[g]) || !aligned16(lut[g]) || !aligned16(out[g])) return AP_EALIGN;
+        const long long segs = (long long)N[g] * (((K[g] >> 5) + kWave - 1) / kWave);
+        if (segs > 0x7fffffffLL) return AP_ELIMIT;
+        items += segs;
+        weights += (long long)N[g] * K[g];
+        mem.qweight[g] = qweight[g];
+        mem.lut[g] = lut[g];
+        mem.out[g] = out[g];
+        mem.N[g] = N[g];
+        mem.K[g] = K[g];
+        mem.item_end[g] = items;
+    }
+    mem.count = count;
     hipStream_t st = static_cast<hipStream_t>(stream);
     drain_stale_error();
     switch (w_bits) {
-        case 3: launch_dequant<3>(qweight, lut, out, N, K, st); break;
-        case 4: launch_dequant<4>(qweight, lut, out, N, K, st); break;
-        case 5: launch_dequant<5>(qweight, lut, out, N, K, st); break;
-        case 6: launch_dequant<6>(qweight, lut, out, N, K, st); break;
-        case 7: launch_dequant<7>(qweight, lut, out, N, K, st); break;
-        default: launch_dequant<8>(qweight, lut, out, N, K, st); break;
+        case 3: launch_dequant<3>(mem, weights, st); break;
+        case 4: launch_dequant<4>(mem, weights, st); break;
+        case 5: launch_dequant<5>(mem, weights, st); break;
+        case 6: launch_dequant<6>(mem, weights, st); break;
+        case 7: launch_dequant<7>(mem, weights, st); break;
+        default: launch_dequant<8>(mem, weights, st); break;
     }
     return launch_status();
 }
@@ -585,37 +604,6 @@ int run_gemvf(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, u
     return launch_status();
 }
 
-// The persistent row-loop GEMV serves rows of a multiple of 64 elements (8-byte plane loads) and up to 4
-// activation rows.
-bool gemvr_fits(int M, int N, int K) {
-    const int W = K >> 5;
-    return M >= 1 && M <= kGemvrMaxM && (W & 1) == 0 && (W + 127) / 128 <= kGemvrMaxSeg;
-}
-
-int run_gemvr(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
-              int w_bits, hipStream_t st) {
-    GemvrGeometry geo;
-    geo.S = ((K >> 5) + 127) / 128;
-    // `gemv_persist_waves` waves per CU, every workgroup walking the same number of rows (+-1), at most 64
-    // (a single-wave workgroup parks one result per lane until its loop ends)
-    int wpc = knob(kGemvPersistWaves);
-    if (wpc < 1) wpc = 1;
-    long long cap = (long long)cu_count() * wpc / geo.S;
-    if (cap < 1) cap = 1;
-    long long rounds = (N + cap - 1) / cap;
-    if (rounds > 64) rounds = 64;
-    geo.grid = (int)((N + rounds - 1) / rounds);
-    switch (w_bits) {
-        case 3: launch_gemvr<3>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 4: launch_gemvr<4>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 5: launch_gemvr<5>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 6: launch_gemvr<6>(M, geo, x, qweight, lut, out, N, K, st); break;
-        case 7: launch_gemvr<7>(M, geo, x, qweight, lut, out, N, K, st); break;
-        default: launch_gemvr<8>(M, geo, x, qweight, lut, out, N, K, st); break;
-    }
-    return launch_status();
-}
-
 int run_gemv4(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
               int w_bits, hipStream_t st) {
     Gemv4Geometry geo;
@@ -671,7 +659,7 @@ struct RouteQuery {
     const int *N;
     int lo, hi;        // fewest / most rows of a member
     long long rows;    // all members together
-    bool fits_persist, fits_fine, fits_stream;  // every member can run that kernel
+    bool fits_fine, fits_stream;  // every member can run that kernel
     const GemvGeometry *geo;                    // of the joint dot-product launch
 };
 
@@ -686,7 +674,6 @@ bool mfma4_fits(const RouteQuery &q) {
 
 // Knobs at 2 force their kernel wherever it fits.  Returns a route or -1.
 int forced_route(const RouteQuery &q) {
-    if (knob(kGemvPersist) >= 2 && q.fits_persist) return AP_ROUTE_PERSIST;  // never a default: slower on every shape
     if (knob(kGemvFine) >= 2 && q.fits_fine) return AP_ROUTE_FINE;
     if (knob(kGemvStream) >= 2 && q.fits_stream) return AP_ROUTE_STREAM;
     return -1;
@@ -789,13 +776,12 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
     // a row longer than one workgroup of the dot-product kernel covers (65536 elements at M <= 2, 32768
     // beyond): the MFMA kernel walks rows of any length
     if (rc == AP_ELIMIT) return all(AP_ROUTE_MFMA16);
-    RouteQuery q = {M, count, K, w_bits, N, N[0], N[0], 0, true, true, true, geo};
+    RouteQuery q = {M, count, K, w_bits, N, N[0], N[0], 0, true, true, geo};
     for (int g = 0; g < count; g++) {
         const uint16_t *o = out ? out[g] : nullptr;
         q.lo = N[g] < q.lo ? N[g] : q.lo;
         q.hi = N[g] > q.hi ? N[g] : q.hi;
         q.rows += N[g];
-        q.fits_persist = q.fits_persist && gemvr_fits(M, N[g], K);
         q.fits_fine = q.fits_fine && gemvf_fits(o, M, N[g], K);
         q.fits_stream = q.fits_stream && gemvp_fits(o, M, N[g], K);
     }
@@ -819,6 +805,60 @@ int plan_matmul(int M, const int *N, int count, int K, int w_bits, uint16_t *con
         }
     }
     return AP_OK;
+}
+
+// Whether the fused GEMM (ap_gemm_kbit) beats dequant_kbit + a library GEMM for `M` activation rows.  Measured on the
+// linear shapes of the Llama-2-7B / Llama-3-8B / 13B / 70B layers at 96..512 activation rows, every bit-width
+// (fused / pair, us):
+//  - always up to 32 activation rows (1.3-4x at 16);
+//  - rows of a multiple of 128 elements (the tiled kernel), linears of at least 4096 rows: up to 128 activation rows at
+//    every bit-width (11008 x 4096, 8 bits: 50 / 58; 28672 x 8192: 189 / 234; 5120 x 13824: 93 / 113); up to 256 at up to
+//    5 bits (11008 x 4096, 4 bits: 58 / 73; 13824 x 5120, 5 bits: 79 / 97), at 6 bits except on linears of more than
+//    16384 rows (28672 x 8192: 263 / 250), at 7 and 8 bits on linears of at most 8192 rows (8192 x 8192, 8 bits:
+//    87 / 116; 5120 x 5120: 56 / 69; 4096 x 11008: 82 / 82; 11008 x 4096: 96 / 66); up to 512 at 3 bits on linears of
+//    at most 8192 rows (4096 x 11008: 87 / 99; 8192 x 8192: 101 / 114; 14336 x 4096: 99 / 90);
+//  - the same rows on linears of 1024..4095 rows: up to 512 activation rows at 3 and 4 bits (1024 x 4096: 11-15 /
+//    18-23; at 6 bits and more the pair wins);
+//  - other row lengths (the K-split kernel only): up to 64 on linears of fewer than 8192 rows, and on larger ones at up
+//    to 5 bits -- except, on rows of more than 4096 elements, from 6 bits on linears of 5120 rows or more and from 5
+//    bits on linears of at most 2048 rows; up to 128 on linears of 4096..8191 rows of at most 4096 elements.
+// Beyond, one table lookup per weight and tile of activation rows costs more than materialising the weight once.
+bool fused_gemm_pays(int M, int N, int K, int b) {
+    if (M <= 32) return true;
+    if ((K & 127) == 0 && M <= 512) {
+        if (N >= 4096) {
+            if (M <= 128) return true;
+            if (M <= 256) return b <= 6 ? (b <= 5 || N <= 16384) : N <= 8192;
+            return b == 3 && N <= 8192;
+        }
+        if (N >= 1024 && b <= 4) return true;
+    }
+    if (M <= 64) {
+        if (K > 4096 && ((b >= 6 && N >= 5120) || (b >= 5 && N <= 2048))) return false;
+        return N < 8192 || b <= 5;
+    }
+    return M <= kGemmMaxM && N >= 4096 && N < 8192 && K <= 4096;
+}
+
+// Whether ONE launch of the tiled GEMM over linears that share their input (ap_gemm_kbit_group) beats calling them one
+// by one, each through whatever fused_gemm_pays picks (q/k/v and gate/up sets of the 7B / 8B / 13B layers at 16..256
+// rows): from 33 rows on -- from 9 where every member has at most 8192 rows (q/k/v of the 7B layer at 16 rows, 3 bits:
+// 16 us against 23; of the 13B layer: 20 against 36); wide members (gate/up) at 9..32 rows are as fast one by one -- up to
+// 128 rows at every bit-width (q/k/v of the 7B layer at 128 rows, 3 bits: 33 us against 44 one by one and 128 for three
+// dequant + GEMM pairs; gate/up at 8 bits: 96 against 115 for the pairs), up to 256 at up to 6 bits (gate/up at 5 bits:
+// 105 against 145) and, at 7 and 8 bits, where every member has fewer than 8192 rows (q/k/v at 8 bits: 94 against 114;
+// gate/up: 145 against 149); up to 512 at 3 bits where no member has more than 8192 rows, as each member alone would.
+bool fused_set_pays(int M, const int *N, int count, int K, int b) {
+    long long sum = 0;
+    int hi = 0;
+    for (int g = 0; g < count; g++) {
+        sum += N[g];
+        hi = N[g] > hi ? N[g] : hi;
+    }
+    if ((K & 127) != 0 || M <= 8 || M > 512 || sum < 4096) return false;
+    if (M > 256) return b == 3 && hi <= 8192;
+    if (M <= 32) return hi <= 8192 && K >= 1024;
+    return M <= 128 || b <= 6 || hi < 8192;
 }
 
 }  // namespace
@@ -945,7 +985,9 @@ int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qwei
     const bool pays = M > 32 || (M > 8 && rows <= 8192 && K >= 1024);
     if (fits && (strided || (count > 1 && mode > 0 && (mode >= 2 || pays))))
         return run_gemmt(tgeo, x, count, qweight, lut, out, N, ldo, M, K, w_bits, static_cast<hipStream_t>(stream));
-    if (strided) return AP_ESHAPE;  // only the tiled kernel writes rows that are not dense
+    // only the tiled kernel writes rows that are not dense: rows it cannot walk at all are a shape error, a size or a
+    // forced tile beyond its geometry a limit (the caller may still ask for dense results)
+    if (strided) return (K & 127) != 0 ? AP_ESHAPE : AP_ELIMIT;
     for (int g = 0; g < count; g++) {
         const int r = ap_gemm_kbit(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, stream);
         if (r != AP_OK) return r;
@@ -1003,13 +1045,30 @@ int ap_matmul_kbit_group(const uint16_t *x, int count, const uint32_t *const *qw
         switch (route[g]) {
             case AP_ROUTE_STREAM: r = run_gemvp(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
             case AP_ROUTE_FINE: r = run_gemvf(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
-            case AP_ROUTE_PERSIST: r = run_gemvr(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
             case AP_ROUTE_MFMA4: r = run_gemv4(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
             default: r = run_gemm(x, qweight[g], lut[g], out[g], M, N[g], K, w_bits, st); break;
         }
         if (r != AP_OK) return r;
     }
     return AP_OK;
+}
+
+int ap_gemm_kbit_pays(int M, int N, int K, int w_bits) {
+    const int rc = check_common(N, K, w_bits);
+    if (rc != AP_OK) return rc;
+    if (M < 1) return AP_EBATCH;
+    return fused_gemm_pays(M, N, K, w_bits) ? 1 : 0;
+}
+
+int ap_gemm_kbit_group_pays(int count, const int *N, int M, int K, int w_bits) {
+    if (!N) return AP_ENULL;
+    if (count < 1 || count > kGemmtMaxGroup) return AP_ELIMIT;
+    for (int g = 0; g < count; g++) {
+        const int rc = check_common(N[g], K, w_bits);
+        if (rc != AP_OK) return rc;
+    }
+    if (M < 1) return AP_EBATCH;
+    return fused_set_pays(M, N, count, K, w_bits) ? 1 : 0;
 }
 
 int ap_matmul_kbit_route(int M, int N, int K, int w_bits, int *route) {

@@ -436,6 +436,17 @@ def main():
             machine["value_over_stream_only"] = round(read_ms / ms_per_step, 4)
         del src, dst
 
+    # what any-precision sells: a 3-bit launch should cost what its bytes cost.  Per shape: time at 3 bits over time at
+    # 8 bits, next to the ratio of the algorithmic bytes (0.34-0.36)
+    low_bits = None
+    if table:
+        low_bits = []
+        for (N, K) in uniq:
+            r3 = next(r for r in table if (r["N"], r["K"], r["w_bits"]) == (N, K, 3))
+            r8 = next(r for r in table if (r["N"], r["K"], r["w_bits"]) == (N, K, 8))
+            low_bits.append({"N": N, "K": K, "t3_over_t8": round(r3["us"] / r8["us"], 3),
+                             "bytes3_over_bytes8": round(r3["bytes"] / r8["bytes"], 3)})
+
     roofline = None
     if table:
         dom = max(table, key=lambda r: r["us"] * r["count_in_step"])
@@ -459,12 +470,13 @@ def main():
         cpu = cpu_baseline(torch, synth, shapes)
 
     # ---- the model-level figure of the same path: batch-1 decode of the Llama-2-7B-shaped model (3 and 8 bits)
-    decode = None
+    decode = prefill = None
     sets_per_shape = {f"{N}x{K}": P.sets for (N, K), P in pools.items()}
     if not args.only_step and not args.no_extras and not args.eager:
         pools.clear()               # the weight pools are no longer needed: make room for the model
         torch.cuda.empty_cache()
         decode = decode_summary(torch)
+        prefill = {"workload": PREFILL_WORKLOAD, "per_w_bits": prefill_rows(torch, synth, reps=3)}
 
     if machine:
         # how much of a step is the fixed cost of its 42 dependent launches, and the rate of the rest
@@ -486,6 +498,7 @@ def main():
         "layers": table,
         "dequant_kbit": dequant_table, "batch_us": batch_table,
         "llama3_8b_batches": llama3, "dequant_layer_set": dequant_layer, "llama2_7b_decode": decode,
+        "llama2_7b_prefill": prefill, "low_bit_time_ratio": low_bits,
     }
     if args.table and table:
         with open(args.table, "w") as f:
@@ -669,8 +682,8 @@ def gemv_kernel_variants(args, torch, _capi, synth):
     gen.manual_seed(0)
     side = torch.cuda.Stream()
     sink = torch.zeros(16, dtype=torch.int32, device="cuda")
-    variants = (("dot", {}), ("fine", {"gemv_fine": 2}), ("stream", {"gemv_stream": 2}), ("persist", {"gemv_persist": 2}))
-    off = {"gemv_fine": 0, "gemv_stream": 0, "gemv_persist": 0}
+    variants = (("dot", {}), ("fine", {"gemv_fine": 2}), ("stream", {"gemv_stream": 2}))
+    off = {"gemv_fine": 0, "gemv_stream": 0}
     bits = (3, 5, 8)
     rows = []
     for N, K in ((4096, 4096), (11008, 4096), (4096, 11008), (28672, 8192)):
@@ -727,7 +740,7 @@ def gemv_kernel_variants(args, torch, _capi, synth):
         "higher_is_better": False, "vs_baseline": None, "data": "synthetic",
         "dtype": "fp16 tables/activations, u32 bitplanes, fp32 accumulate",
         "config": {"workload": "4096x4096, 11008x4096, 4096x11008, 28672x8192 at w_bits 3, 5, 8, batch 1; each of the "
-                               "dot / fine / stream / persist kernels forced through ap_set_tuning; cold weight sets; "
+                               "dot / fine / stream kernels forced through ap_set_tuning; cold weight sets; "
                                + ("eager launches" if args.eager else "HIP graphs")},
         "value": None, "kernels": rows}))
 
@@ -1046,15 +1059,16 @@ def _llama2_7b_config():
                        tie_word_embeddings=False)
 
 
-def decode_summary(torch, prompt_len=128, new_tokens=96):
-    """tokens/s of the graph-replayed decode step on a random-init Llama-2-7B-shaped model after a
-    128-token prompt, at 3 and 8 bits (the full sweep is --workload llama2_7b_decode)."""
+def decode_summary(torch, prompt_len=128, new_tokens=256):
+    """tokens/s of the graph-replayed decode step on a random-init Llama-2-7B-shaped model: 256 tokens after a
+    128-token prompt at every w_bits 3..8, the loop of the reference's demo.py:59-80 (--workload llama2_7b_decode
+    adds the prompt time and the other decode modes)."""
     from any_precision_amd import AnyPrecisionForCausalLM, GraphDecoder
     model = AnyPrecisionForCausalLM.from_config(_llama2_7b_config(), seed=0, device="cuda")
     dec = GraphDecoder(model, max_len=prompt_len + new_tokens + 8)
     ids = torch.randint(0, 32000, (prompt_len,), generator=torch.Generator().manual_seed(0)).cuda()
     rows = []
-    for b in (3, 8):
+    for b in BITS:
         dec.prefill(ids, b)
         dec.capture(b)
         dec.decode(8, b)
@@ -1103,7 +1117,7 @@ def decode_tokens(args, torch, _capi, synth):
         # the launch rules were fitted to launches timed alone; this times the whole step with one rule overridden at a time
         overrides = [("rows_1", {"gemv_rows": 1}), ("rows_2", {"gemv_rows": 2}), ("rows_4", {"gemv_rows": 4}),
                      ("no_stream", {"gemv_stream": 0}), ("stream_everywhere", {"gemv_stream": 2}), ("no_fine", {"gemv_fine": 0}),
-                     ("fine_everywhere", {"gemv_fine": 2}), ("no_persist", {"gemv_persist": 0}), ("persist_everywhere", {"gemv_persist": 2}),
+                     ("fine_everywhere", {"gemv_fine": 2}),
                      ("target_waves_8192", {"gemv_target_waves": 8192}), ("target_waves_32768", {"gemv_target_waves": 32768})]
 
         def tokens_per_s(b, knobs):
@@ -1210,10 +1224,14 @@ def decode_tokens(args, torch, _capi, synth):
 
 
 
-def prefill_linears(args, torch, _capi, synth):
-    """The seven linears of a Llama-2-7B layer on M = 32 x 512 activation rows through AnyPrecisionLinear's
-    large-batch branch: dequant_kbit to fp16, then the library GEMM.  Reports the share of the dequant, and beside it
-    the same rows through ap_gemm_kbit (the tiled fused kernel, one launch per linear)."""
+MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 matrix-core peak of MI355X
+
+
+def prefill_rows(torch, synth, bits=(3, 8), reps=5):
+    """The seven linears of a Llama-2-7B layer on M = 32 x 512 = 16384 activation rows, two routes per w_bits:
+    the module's forward (AnyPrecisionLinear's branch for many rows: dequant_kbit to fp16, then the library GEMM --
+    the reference's AnyPrecisionLinear.py:60-62) and ap_gemm_kbit (the fused tiled dequant -> LDS -> MFMA kernel, one
+    launch per linear).  ms per layer set, TFLOP/s and the fraction of the 2.5 PFLOP/s fp16 matrix-core peak."""
     from any_precision_amd import AnyPrecisionLinear
     import any_precision_ext as ext
     gen = torch.Generator(device="cuda")
@@ -1222,43 +1240,54 @@ def prefill_linears(args, torch, _capi, synth):
     side = torch.cuda.Stream()
     rows = []
     with torch.inference_mode():
-        for b in (3, 8):
+        for b in bits:
             t_total = t_deq = t_fused = flops = 0.0
             for name, N, K in synth.LLAMA2_7B_LAYER:
-                lin = AnyPrecisionLinear(K, N, list(range(3, 9)), bias=False, device="cuda", dtype=torch.float16)
+                lin = AnyPrecisionLinear(K, N, [b], bias=False, device="cuda", dtype=torch.float16)
                 lin.qweight.copy_(torch.randint(-2**31, 2**31 - 1, lin.qweight.shape, dtype=torch.int32, device="cuda",
                                                 generator=gen))
                 lin._buffers[f"lut{b}"].copy_(torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02,
                                                          dim=1).values.half())
                 x = torch.randn((M, K), device="cuda", generator=gen).half()
 
-                def run(fn, reps=5):
+                def run(fn, n):
                     with torch.cuda.stream(side):
                         fn()
                         side.synchronize()
                         a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                         a0.record(side)
-                        for _ in range(reps):
+                        for _ in range(n):
                             fn()
                         a1.record(side)
                         side.synchronize()
-                    return a0.elapsed_time(a1) / reps
-                t_total += run(lambda: lin(x, precision=b))
-                t_deq += run(lambda: ext.dequant_kbit(lin.qweight, lin._buffers[f"lut{b}"], b))
-                # the same rows through the fused tiled GEMM in one launch, for the record (it is not what the module uses here)
-                t_fused += run(lambda: ext.gemm_kbit(x, lin.qweight, lin._buffers[f"lut{b}"], b), reps=2)
+                    return a0.elapsed_time(a1) / n
+                t_total += run(lambda: lin(x, precision=b), reps)
+                t_deq += run(lambda: ext.dequant_kbit(lin.qweight, lin._buffers[f"lut{b}"], b), reps)
+                t_fused += run(lambda: ext.gemm_kbit(x, lin.qweight, lin._buffers[f"lut{b}"], b), max(2, reps // 2))
                 flops += 2.0 * M * N * K
                 del lin, x
             rows.append({"w_bits": b, "ms_per_layer_linears": round(t_total, 3), "ms_dequant": round(t_deq, 3),
                          "dequant_share": round(t_deq / t_total, 4), "TFLOPs": round(flops / t_total / 1e9, 1),
-                         "fused_tiled_gemm_ms": round(t_fused, 3), "fused_tiled_gemm_TFLOPs": round(flops / t_fused / 1e9, 1)})
+                         "frac_of_mfma_peak": round(flops / t_total / 1e9 / MFMA_PEAK_TFLOPS, 4),
+                         "fused_tiled_gemm_ms": round(t_fused, 3), "fused_tiled_gemm_TFLOPs": round(flops / t_fused / 1e9, 1),
+                         "fused_tiled_gemm_frac_of_mfma_peak": round(flops / t_fused / 1e9 / MFMA_PEAK_TFLOPS, 4)})
+    torch.cuda.empty_cache()
+    return rows
+
+
+PREFILL_WORKLOAD = ("7 linears of a Llama-2-7B decoder layer, M = 32 x 512 = 16384 activation rows, eager launches: the "
+                    "module's route (dequant_kbit + torch.matmul per call, weight rebuilt on every call) and, beside it, "
+                    "ap_gemm_kbit (fused tiled kernel)")
+
+
+def prefill_linears(args, torch, _capi, synth):
+    rows = prefill_rows(torch, synth)
     print(json.dumps({
         "metric": "prefill linears TFLOP/s, Llama-2-7B layer set, 16384 activation rows",
         "value": round(sum(r["TFLOPs"] for r in rows) / len(rows), 1), "unit": "TFLOP/s", "n_gpus": 1,
         "higher_is_better": True, "vs_baseline": None, "dtype": "fp16 (library GEMM) on dequantised weights",
         "data": "synthetic",
-        "config": {"workload": "7 linears of a Llama-2-7B decoder layer, M = 32 x 512 rows, dequant_kbit + "
-                               "torch.matmul per call (weight rebuilt on every call), eager launches"},
+        "config": {"workload": PREFILL_WORKLOAD},
         "per_w_bits": rows}))
 
 

@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define AP_ABI_VERSION 7
+#define AP_ABI_VERSION 8
 
 enum {
     AP_OK = 0,
@@ -52,6 +52,16 @@ enum {
  * out[n,k] = lut[n, code[n,k] >> (P - w_bits)], bit-exact copy of table entries. */
 int ap_dequant_kbit(const uint32_t *qweight, const uint16_t *lut, uint16_t *out,
                     int N, int K, int w_bits, void *stream);
+
+/* ap_dequant_kbit for `count` (1..8) linears of any shapes at one w_bits in ONE launch:
+ * out[g][N[g], K[g]] = dequant(qweight[g], lut[g]).  The arrays are host arrays of `count` device
+ * pointers / sizes.  For dequantising a whole decoder layer (seven linears) or a whole checkpoint
+ * (config "full weight set"): the reference launches dequant_kbit_store once per linear
+ * (main.cu:82-84); here the 64-word segments of all members share one grid, so the fixed cost and
+ * the tail of a launch are paid once.  Results are bit-identical to `count` calls of ap_dequant_kbit.
+ * AP_ELIMIT for count outside 1..8. */
+int ap_dequant_kbit_group(int count, const uint32_t *const *qweight, const uint16_t *const *lut,
+                          uint16_t *const *out, const int *N, const int *K, int w_bits, void *stream);
 
 /* Replaces matmul_kbit(in, qweight, lut, w_bits) -> Tensor[..., N]
  * (main.cu:93-143, kernel matmul.cuh:16-167).  1 <= M <= 8 as in the
@@ -107,11 +117,20 @@ int ap_gemm_kbit(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut
  * ldo (may be NULL: dense results) gives the distance in elements between consecutive rows of each
  * out[g], so that the results can be written side by side into one [M, sum N] array (out[g] = its
  * column offset, ldo[g] = sum N); results that are not dense need the tiled kernel: AP_ESHAPE if
- * K % 128 != 0 then.  No counterpart in the reference (its fuse_layers hook is a stub,
+ * K % 128 != 0 then, AP_ELIMIT if M * K exceeds its 32-bit offsets (ask for dense results instead).  No counterpart in the reference (its fuse_layers hook is a stub,
  * AnyPrecisionForCausalLM.py:168-172).  AP_ELIMIT for count outside 1..4. */
 int ap_gemm_kbit_group(const uint16_t *x, int count, const uint32_t *const *qweight,
                        const uint16_t *const *lut, uint16_t *const *out, const int *N,
                        const long long *ldo, int M, int K, int w_bits, void *stream);
+
+/* Where the fused GEMM is the faster way to compute x . dequant(W)^T, from this library's measurements on
+ * MI355X: ap_gemm_kbit_pays returns 1 if ap_gemm_kbit beats ap_dequant_kbit + a library fp16 GEMM for M
+ * activation rows on an [N, K] linear at w_bits, 0 if the pair wins (the reference always takes the pair
+ * above 8 rows, AnyPrecisionLinear.py:60-62); ap_gemm_kbit_group_pays the same for ONE ap_gemm_kbit_group
+ * launch over `count` linears against calling them one by one.  The host module asks these instead of
+ * keeping thresholds of its own.  Negative argument errors as for ap_gemm_kbit. */
+int ap_gemm_kbit_pays(int M, int N, int K, int w_bits);
+int ap_gemm_kbit_group_pays(int count, const int *N, int M, int K, int w_bits);
 
 /* Human-readable text for a return code of the functions above. */
 const char *ap_strerror(int code);
@@ -131,9 +150,8 @@ enum {
     AP_ROUTE_DOT = 0,     /* gemv_kbit_kernel: one, two or four rows per workgroup                      */
     AP_ROUTE_STREAM = 1,  /* gemvp_kbit_kernel: row pairs, 16-byte plane loads, few long waves           */
     AP_ROUTE_FINE = 2,    /* gemvf_kbit_kernel: one workgroup per row pair, 8-byte plane loads           */
-    AP_ROUTE_PERSIST = 3, /* gemvr_kbit_kernel: persistent row loop (only when forced)                   */
-    AP_ROUTE_MFMA4 = 4,   /* gemv4_kbit_kernel: 4x4x4 matrix-core kernel                                 */
-    AP_ROUTE_MFMA16 = 5   /* gemm_kbit_kernel: 16x16x32 matrix-core kernel                               */
+    AP_ROUTE_MFMA4 = 3,   /* gemv4_kbit_kernel: 4x4x4 matrix-core kernel                                 */
+    AP_ROUTE_MFMA16 = 4   /* gemm_kbit_kernel: 16x16x32 matrix-core kernel                               */
 };
 int ap_matmul_kbit_route(int M, int N, int K, int w_bits, int *route);
 /* The same for a set of `count` linears given to ap_matmul_kbit_group: route[g] per member (all AP_ROUTE_DOT = one
@@ -147,8 +165,10 @@ int ap_matmul_kbit_group_route(int count, const int *N, int M, int K, int w_bits
  * beyond the 1e-2 bar of the entry points; the defaults are what measured fastest.  Names:
  * gemv_target_waves, gemv_rows, gemv_wpl, dequant_blocks_per_cu, matmul_mfma_from, gemm_split,
  * matmul_mfma4, gemv4_groups, gemm_rb2, gemv_stream, gemv_stream_waves, gemv_fine,
- * gemv_persist, gemv_persist_waves, gemm_walk, gemm_walk_wgs, gemm_tiled, gemm_tile, gemm_tile_split.  Returns AP_OK, AP_ENULL
- * or AP_EKNOB. */
+ * gemm_walk, gemm_walk_wgs, gemm_tiled, gemm_tile, gemm_tile_split.  Returns AP_OK, AP_ENULL or AP_EKNOB.
+ * For tests and measurements only: the knobs are plain process-wide integers, NOT thread-safe against
+ * concurrent launches (a launch that races with a change sees either value); a serving process leaves
+ * them alone. */
 int ap_set_tuning(const char *name, int value);
 int ap_get_tuning(const char *name, int *value);
 

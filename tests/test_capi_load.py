@@ -131,8 +131,7 @@ def test_tuning_knobs_need_no_gpu():
     with pytest.raises(ValueError):
         _capi.get_tuning("no_such_knob")
     for name in ("gemv_target_waves", "gemv_rows", "gemv_wpl", "dequant_blocks_per_cu", "matmul_mfma_from", "gemm_split",
-                 "matmul_mfma4", "gemv4_groups", "gemm_rb2", "gemv_stream", "gemv_stream_waves", "gemv_fine",
-                 "gemv_persist", "gemv_persist_waves"):
+                 "matmul_mfma4", "gemv4_groups", "gemm_rb2", "gemv_stream", "gemv_stream_waves", "gemv_fine"):
         before = _capi.get_tuning(name)
         with _capi.tuning(**{name: before + 3}):
             assert _capi.get_tuning(name) == before + 3
@@ -174,9 +173,9 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_route(1, 8, 32 * 64 * 2 * 17, 4) == "mfma16"      # longer than a workgroup covers
     with _capi.tuning(gemv_stream=0, gemv_fine=0):
         assert _capi.matmul_route(1, 11008, 4096, 3) == "dot"
-    with _capi.tuning(gemv_persist=2):
-        assert _capi.matmul_route(3, 64, 4096, 5) == "persist"
-        assert _capi.matmul_route(3, 64, 4128, 5) != "persist"            # rows must be a multiple of 64 elements
+    with _capi.tuning(gemv_stream=2):
+        assert _capi.matmul_route(3, 64, 4096, 5) == "stream"
+        assert _capi.matmul_route(3, 64, 4128, 5) != "stream"             # rows must be a multiple of 128 elements
     with _capi.tuning(gemv_fine=2):
         assert _capi.matmul_route(1, 63, 4096, 5) == "dot"                # odd row count: not served
     with pytest.raises(ValueError):

@@ -50,12 +50,13 @@ def test_cpu_tensors_are_rejected_not_computed():
 
 def test_fused_gemm_dispatch_rule():
     """Where AnyPrecisionLinear takes the fused GEMM instead of dequant + matmul (the reference sends everything above
-    8 rows to dequant + matmul, AnyPrecisionLinear.py:60-62): the rule as it was fitted to the measured sweep."""
+    8 rows to dequant + matmul, AnyPrecisionLinear.py:60-62): the rule as it was fitted to the measured sweep.  The
+    thresholds live in the library (ap_gemm_kbit_pays); the module only asks."""
     from any_precision_amd.linear import fused_gemm_pays
-    assert all(fused_gemm_pays(m, n, b) for m in (9, 32) for n in (4096, 14336) for b in (3, 8))
-    # rows the tiled kernel does not take (not a multiple of 128 elements, or unknown): the K-split kernel's crossovers
-    assert fused_gemm_pays(64, 4096, 8) and fused_gemm_pays(64, 14336, 5) and not fused_gemm_pays(64, 14336, 6)
-    assert not fused_gemm_pays(65, 4096, 5) and not fused_gemm_pays(129, 4096, 6, 4000) and fused_gemm_pays(128, 4096, 6, 4000)
+    assert all(fused_gemm_pays(m, n, b, k) for m in (9, 32) for n in (4096, 14336) for b in (3, 8) for k in (4000, 4096))
+    # rows the tiled kernel does not take (not a multiple of 128 elements): the K-split kernel's crossovers
+    assert fused_gemm_pays(64, 4096, 8, 4000) and fused_gemm_pays(64, 14336, 5, 4000) and not fused_gemm_pays(64, 14336, 6, 4000)
+    assert not fused_gemm_pays(65, 4096, 5, 8224) and not fused_gemm_pays(129, 4096, 6, 4000) and fused_gemm_pays(128, 4096, 6, 4000)
     assert not fused_gemm_pays(64, 14336, 8, 4000) and not fused_gemm_pays(200, 4096, 3, 4000)
     assert fused_gemm_pays(64, 1024, 8, 4096) and not fused_gemm_pays(64, 1024, 5, 8192)        # narrow, long rows
     # the tiled kernel, linears of at least 4096 rows: every bit-width up to 128 activation rows
@@ -71,3 +72,5 @@ def test_fused_gemm_dispatch_rule():
     # linears of 1024..4095 rows: 3 and 4 bits up to 512
     assert fused_gemm_pays(100, 1024, 3, 4096) and fused_gemm_pays(512, 1024, 4, 8192) and not fused_gemm_pays(100, 1024, 5, 4096)
     assert not fused_gemm_pays(100, 512, 3, 4096)
+    with pytest.raises(ValueError):
+        fused_gemm_pays(16, 4096, 3, 4097)                # not a row length the layout has

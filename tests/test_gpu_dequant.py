@@ -112,3 +112,43 @@ def test_idempotent_and_row_independent(ext):
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
     sub = ext.dequant_kbit(q[:, 1000:1512].contiguous(), luts[7][1000:1512].contiguous(), 7)
     assert torch.equal(sub.view(torch.int16), a[1000:1512].view(torch.int16))
+
+
+def test_grouped_launch_is_bit_identical_to_the_separate_calls(ext, oracle):
+    """dequant_kbit_group: up to eight linears of different shapes in one launch (ragged rows, tail chunks, a
+    member of one segment, members larger than a grid round) against the oracle and the single calls."""
+    from any_precision_amd import _capi
+    shapes = [(13, 1056), (1, 32), (130, 992), (4, 2080), (640, 4096), (96, 11008), (7, 32), (33, 1024)]
+    layers = [make(N, K, seed=3 * N + K) for N, K in shapes]
+    on_gpu = [layer_to_gpu(L) for L in layers]
+    for b in range(3, 9):
+        for count in (1, 2, 7, 8):
+            print(f"dequant group b={b} count={count}", flush=True)
+            got = ext.dequant_kbit_group([q for q, _ in on_gpu[:count]], [t[b] for _, t in on_gpu[:count]], b)
+            assert len(got) == count
+            for g, (L, (q, luts)) in enumerate(zip(layers[:count], on_gpu[:count])):
+                assert_bit_exact(got[g], oracle.dequant_kbit(L.qweight, L.luts[b], b), f"member {g} b={b} count={count}")
+                assert torch.equal(got[g].view(torch.int16), ext.dequant_kbit(q, luts[b], b).view(torch.int16))
+    # a small grid (one workgroup per CU): every wave strides through several members
+    with _capi.tuning(dequant_blocks_per_cu=1):
+        got = ext.dequant_kbit_group([q for q, _ in on_gpu], [t[5] for _, t in on_gpu], 5)
+    for g, L in enumerate(layers):
+        assert_bit_exact(got[g], oracle.dequant_kbit(L.qweight, L.luts[5], 5), f"strided member {g}")
+    with pytest.raises(ValueError):
+        ext.dequant_kbit_group([on_gpu[0][0]] * 9, [on_gpu[0][1][3]] * 9, 3)
+
+
+def test_grouped_launch_over_a_decoder_layer_set(ext):
+    """The seven linears of a Llama-2-7B layer in one launch against the single calls, bit for bit (random planes)."""
+    from any_precision_amd import synth
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(11)
+    qs = [torch.randint(-2**31, 2**31 - 1, (8, N, K // 32), dtype=torch.int32, device="cuda", generator=gen)
+          for _, N, K in synth.LLAMA2_7B_LAYER]
+    for b in (3, 8):
+        ts = [torch.sort(torch.randn((N, 1 << b), device="cuda", generator=gen) * 0.02, dim=1).values.half()
+              for _, N, K in synth.LLAMA2_7B_LAYER]
+        got = ext.dequant_kbit_group(qs, ts, b)
+        for g, (q, t) in enumerate(zip(qs, ts)):
+            assert torch.equal(got[g].view(torch.int16), ext.dequant_kbit(q, t, b).view(torch.int16)), f"member {g} b={b}"
+        del got

@@ -218,10 +218,10 @@ WAVE_SPLIT_SHAPES = [(2, 64), (130, 128), (34, 1088), (10, 2048), (64, 4096), (2
                      (6, 28672), (1030, 1024)]
 
 
-@pytest.mark.parametrize("knob", ["gemv_fine", "gemv_stream", "gemv_persist"])
+@pytest.mark.parametrize("knob", ["gemv_fine", "gemv_stream"])
 def test_the_other_splits_of_the_work_over_waves_agree_with_the_oracle(ext, oracle, knob):
-    """Three more dot-product kernels serve 1..4 activation rows (fine-grained row pairs, row-streaming
-    row pairs with 16-byte loads, persistent row loop); the default rule uses them on a few wide shapes
+    """Two more dot-product kernels serve 1..4 activation rows (fine-grained row pairs, row-streaming
+    row pairs with 16-byte loads); the default rule uses them on a few wide shapes
     only, so each is forced (knob = 2) over ragged and tail shapes, every bit-width, M = 1..4, and checked
     against the oracle at the path's 1e-2 bar.  Shapes a kernel does not serve (odd row counts, rows that
     are not a multiple of 64 / 128 elements) must fall through to the default kernels."""
@@ -241,7 +241,7 @@ def test_the_other_splits_of_the_work_over_waves_agree_with_the_oracle(ext, orac
                     assert_close_gemv(got, want, f"{knob} waves={waves} N={N} K={K} b={b} M={M}")
 
 
-@pytest.mark.parametrize("knob", ["gemv_fine", "gemv_stream", "gemv_persist"])
+@pytest.mark.parametrize("knob", ["gemv_fine", "gemv_stream"])
 def test_the_other_splits_are_exact_on_one_hot_activations_and_deterministic(ext, oracle, knob):
     """x = e_k picks column k of the dequantised weight: the fp16 result must be that table entry bit for
     bit (covers the word -> element mapping of every lane, tail chunk included); two runs must agree."""
