@@ -35,7 +35,7 @@ def parse_args():
     ap.add_argument("--workload", default="llama2_7b_layer_batch1",
                     choices=("llama2_7b_layer_batch1", "llama3_8b_layer_batches", "llama2_7b_dequant_full_model",
                              "llama2_7b_decode", "llama2_7b_prefill", "llama2_7b_gemm_rows", "gemv_kernel_variants",
-                             "routing_audit"),
+                             "routing_audit", "profile_set"),
                     help="default: the headline (42 GEMVs of a Llama-2-7B layer at batch 1).  "
                          "llama3_8b_layer_batches: matmul_kbit on the Llama-3-8B shapes at M = 1, 2, 4, 8.  "
                          "llama2_7b_dequant_full_model: dequant_kbit over all 224 linears of Llama-2-7B.  "
@@ -49,6 +49,10 @@ def parse_args():
                          "gemv_kernel_variants: the four dot-product GEMV kernels forced in turn (tuning knobs) on "
                          "the headline shapes and on 28672 x 8192, batch 1, beside the read-only stream; with "
                          "--eager the launches go out one by one (the form rocprofv3 counter runs need).  "
+                         "profile_set: one eager launch list for rocprofv3 runs -- every kernel the default routes of the "
+                         "Llama-2-7B layer use: the 18 single GEMVs, the q/k/v and gate/up group launches, the SwiGLU pair "
+                         "launch, dequant_kbit per linear and per layer set, the fused GEMM at 16 and 16384 rows; "
+                         "--kernel-reps launches per case on rotating weight sets, a manifest of the cases on stdout.  "
                          "routing_audit: for the linears of the models named by --audit-models, at 1..8 activation "
                          "rows and 3, 4, 5, 8 bits, the time of what ap_matmul_kbit launches by default beside every "
                          "kernel and geometry the tuning knobs can force: where is the default not the fastest.")
@@ -116,6 +120,8 @@ def main():
         return gemv_kernel_variants(args, torch, _capi, synth)
     if args.workload == "routing_audit":
         return routing_audit(args, torch, _capi, synth)
+    if args.workload == "profile_set":
+        return profile_set(args, torch, _capi, synth)
     if args.workload == "llama2_7b_gemm_rows":
         return gemm_rows(args, torch, _capi, synth)
     if args.workload == "llama2_7b_decode":
@@ -961,6 +967,93 @@ def routing_audit(args, torch, _capi, synth):
                                + "; cold weight sets; HIP graphs; alternatives forced through ap_set_tuning"},
         "cases": len(cases), "worst_excess": max((l["excess"] for l in losses), default=0.0),
         "losses": sorted(losses, key=lambda l: -l["excess"]), "all_cases": cases}))
+
+
+def profile_set(args, torch, _capi, synth):
+    """Eager launches of every kernel the default routes of the Llama-2-7B layer use, `--kernel-reps` per case on
+    rotating (cold) weight sets, each case exactly one kernel dispatch per launch; prints the ordered manifest of the
+    cases so that the dispatches of a rocprofv3 trace or counter run can be attributed (the library's kernels appear
+    in launch order; with --calibrate-copy three 256 MiB torch.add launches of known traffic come first)."""
+    lib = _capi.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0)
+    reps = max(1, min(args.kernel_reps, 8))
+    shapes = sorted({(N, K) for _, N, K in synth.LLAMA2_7B_LAYER})
+    pools = {(N, K): WeightPool(torch, N, K, max(reps, 3), gen) for N, K in shapes}
+    x1 = {K: torch.randn((1, K), device="cuda", generator=gen).half() for K in (4096, 11008)}
+    out = torch.empty((16, 3 * 11008), dtype=torch.float16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    manifest = []
+
+    def case(label, launch):
+        for i in range(reps):
+            rc = launch(i)
+            if rc not in (0, None):
+                raise RuntimeError(f"{label}: {_capi.strerror(rc)}")
+        torch.cuda.synchronize()
+        manifest.append({"case": label, "dispatches": reps})
+
+    if args.calibrate_copy:
+        src = torch.ones(64 << 20, dtype=torch.int32, device="cuda")      # 256 MiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)      # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+    for b in BITS:
+        for N, K in shapes:
+            P = pools[(N, K)]
+            case(f"matmul_kbit {N}x{K} M=1 b={b} [{_capi.matmul_route(1, N, K, b)}]",
+                 lambda i: lib.ap_matmul_kbit(x1[K].data_ptr(), P.qweight[i].data_ptr(), P.luts[b][i].data_ptr(), out.data_ptr(),
+                                              1, N, K, b, st))
+    for b in BITS:
+        P = pools[(4096, 4096)]
+        case(f"matmul_kbit_group q,k,v 3x4096x4096 M=1 b={b}",
+             lambda i: _capi.matmul_group(x1[4096].data_ptr(), [P.qweight[(i + g) % P.sets].data_ptr() for g in range(3)],
+                                          [P.luts[b][(i + g) % P.sets].data_ptr() for g in range(3)],
+                                          [out.data_ptr() + 2 * 4096 * g for g in range(3)], [4096] * 3, 1, 4096, b, st))
+        P = pools[(11008, 4096)]
+        case(f"matmul_kbit_group gate,up 2x11008x4096 M=1 b={b}",
+             lambda i: _capi.matmul_group(x1[4096].data_ptr(), [P.qweight[(i + g) % P.sets].data_ptr() for g in range(2)],
+                                          [P.luts[b][(i + g) % P.sets].data_ptr() for g in range(2)],
+                                          [out.data_ptr() + 2 * 11008 * g for g in range(2)], [11008] * 2, 1, 4096, b, st))
+        case(f"matmul_kbit_swiglu gate,up 2x11008x4096 M=1 b={b}",
+             lambda i: lib.ap_matmul_kbit_swiglu(x1[4096].data_ptr(), P.qweight[i].data_ptr(), P.luts[b][i].data_ptr(),
+                                                 P.qweight[(i + 1) % P.sets].data_ptr(), P.luts[b][(i + 1) % P.sets].data_ptr(),
+                                                 out.data_ptr(), 1, 11008, 4096, b, st))
+    # dequant: per linear and the seven linears of a layer in one launch
+    wout = {(N, K): torch.empty((2, N, K), dtype=torch.float16, device="cuda") for N, K in shapes}
+    for b in BITS:
+        for N, K in shapes:
+            P = pools[(N, K)]
+            case(f"dequant_kbit {N}x{K} b={b}",
+                 lambda i: lib.ap_dequant_kbit(P.qweight[i].data_ptr(), P.luts[b][i].data_ptr(), wout[(N, K)][i & 1].data_ptr(), N, K, b, st))
+    layer = [(N, K) for _, N, K in synth.LLAMA2_7B_LAYER]
+    wlayer = [torch.empty((N, K), dtype=torch.float16, device="cuda") for N, K in layer]
+    for b in (3, 8):
+        case(f"dequant_kbit_group 7 linears of a layer b={b}",
+             lambda i: _capi.dequant_group([pools[s].qweight[(i + g) % pools[s].sets].data_ptr() for g, s in enumerate(layer)],
+                                           [pools[s].luts[b][(i + g) % pools[s].sets].data_ptr() for g, s in enumerate(layer)],
+                                           [w.data_ptr() for w in wlayer], [N for N, _ in layer], [K for _, K in layer], b, st))
+    del wout, wlayer
+    # fused GEMM: 16 rows (K-split kernel) and 16384 rows (tiled kernel, one launch)
+    x16 = torch.randn((16, 4096), device="cuda", generator=gen).half()
+    xp = torch.randn((32 * 512, 4096), device="cuda", generator=gen).half()
+    outp = torch.empty((32 * 512, 11008), dtype=torch.float16, device="cuda")
+    for b in (3, 8):
+        for N, K in ((4096, 4096), (11008, 4096)):
+            P = pools[(N, K)]
+            case(f"gemm_kbit {N}x{K} M=16 b={b}",
+                 lambda i: lib.ap_gemm_kbit(x16.data_ptr(), P.qweight[i].data_ptr(), P.luts[b][i].data_ptr(), outp.data_ptr(),
+                                            16, N, K, b, st))
+            case(f"gemm_kbit {N}x{K} M=16384 b={b}",
+                 lambda i: lib.ap_gemm_kbit(xp.data_ptr(), P.qweight[i].data_ptr(), P.luts[b][i].data_ptr(), outp.data_ptr(),
+                                            32 * 512, N, K, b, st))
+    print(json.dumps({"metric": "profile launch list (no timing)", "value": None, "unit": None, "n_gpus": 1,
+                      "higher_is_better": True, "vs_baseline": None, "data": "synthetic",
+                      "config": {"workload": "every kernel of the default routes of the Llama-2-7B layer, eager, "
+                                             f"{reps} launches per case"},
+                      "calibration_dispatches": 3 if args.calibrate_copy else 0, "manifest": manifest}))
 
 
 def gemm_rows(args, torch, _capi, synth):
