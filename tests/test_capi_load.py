@@ -110,6 +110,33 @@ def test_gemm_group_argument_errors_need_no_gpu():
     assert call(t=[fake, fake + 2]) == _capi.AP_EALIGN and call(x=fake + 8) == _capi.AP_EALIGN
 
 
+def test_dequant_group_and_pays_argument_errors_need_no_gpu():
+    """ap_dequant_kbit_group, ap_gemm_kbit_pays and ap_gemm_kbit_group_pays check their arguments before any HIP call."""
+    import ctypes
+    from any_precision_amd import _capi
+    fake = 4096
+    call = lambda **kw: _capi.dequant_group(kw.get("q", [fake, fake]), kw.get("t", [fake, fake]), kw.get("o", [fake, fake]),
+                                            kw.get("N", [64, 8]), kw.get("K", [128, 2080]), kw.get("b", 3), 0)
+    assert call(q=[fake, None]) == _capi.AP_ENULL and call(o=[None, fake]) == _capi.AP_ENULL
+    assert call(q=[fake] * 9, t=[fake] * 9, o=[fake] * 9, N=[64] * 9, K=[128] * 9) == _capi.AP_ELIMIT
+    assert _capi.lib.ap_dequant_kbit_group(0, None, None, None, None, None, 3, None) == _capi.AP_ENULL
+    assert call(b=9) == _capi.AP_EBITS
+    assert call(K=[128, 100]) == _capi.AP_ESHAPE and call(N=[64, 0]) == _capi.AP_ESHAPE
+    assert call(t=[fake, fake + 2]) == _capi.AP_EALIGN and call(o=[fake + 8, fake]) == _capi.AP_EALIGN
+    assert _capi.lib.ap_dequant_kbit(None, fake, fake, 8, 64, 3, None) == _capi.AP_ENULL      # the single call is a set of one
+    assert _capi.lib.ap_gemm_kbit_pays(16, 4096, 4096, 3) == 1 and _capi.lib.ap_gemm_kbit_pays(16384, 4096, 4096, 3) == 0
+    assert _capi.lib.ap_gemm_kbit_pays(0, 4096, 4096, 3) == _capi.AP_EBATCH
+    assert _capi.lib.ap_gemm_kbit_pays(16, 4096, 4100, 3) == _capi.AP_ESHAPE
+    assert _capi.lib.ap_gemm_kbit_pays(16, 4096, 4096, 2) == _capi.AP_EBITS
+    three = (ctypes.c_int * 3)(4096, 4096, 4096)
+    assert _capi.lib.ap_gemm_kbit_group_pays(3, three, 128, 4096, 3) == 1
+    assert _capi.lib.ap_gemm_kbit_group_pays(3, three, 8, 4096, 3) == 0
+    assert _capi.lib.ap_gemm_kbit_group_pays(5, three, 128, 4096, 3) == _capi.AP_ELIMIT
+    assert _capi.lib.ap_gemm_kbit_group_pays(3, None, 128, 4096, 3) == _capi.AP_ENULL
+    with pytest.raises(ValueError):
+        _capi.gemm_pays(16, 0, 4096, 3)
+
+
 def test_geometry_covers_rows_and_words():
     from any_precision_amd import _capi
     for M in (1, 2, 4, 8):

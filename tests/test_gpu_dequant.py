@@ -152,3 +152,28 @@ def test_grouped_launch_over_a_decoder_layer_set(ext):
         for g, (q, t) in enumerate(zip(qs, ts)):
             assert torch.equal(got[g].view(torch.int16), ext.dequant_kbit(q, t, b).view(torch.int16)), f"member {g} b={b}"
         del got
+
+
+def test_grouped_launch_replays_in_a_graph(ext):
+    """One ap_dequant_kbit_group launch captured in a HIP graph (members travel as kernel arguments: nothing to copy at
+    replay) against the eager result on every replay, with eager work and synchronisations between the replays."""
+    shapes = [(96, 4096), (64, 11008), (33, 1024)]
+    layers = [make(N, K, seed=7 * N + K) for N, K in shapes]
+    on_gpu = [layer_to_gpu(L) for L in layers]
+    b = 5
+    qs, ts = [q for q, _ in on_gpu], [t[b] for _, t in on_gpu]
+    want = ext.dequant_kbit_group(qs, ts, b)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            got = ext.dequant_kbit_group(qs, ts, b)
+    for rep in range(3):
+        for g in got:
+            g.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for g, (a, w) in enumerate(zip(got, want)):
+            assert torch.equal(a.view(torch.int16), w.view(torch.int16)), f"replay {rep} member {g}"
+        _ = ext.dequant_kbit(qs[0], ts[0], b)      # eager work between the replays
