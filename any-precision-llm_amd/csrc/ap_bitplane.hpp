@@ -106,58 +106,10 @@ AP_HD void planes_to_indices(const uint32_t (&q)[BITS], uint32_t (&idx)[8]) {
     for (int e = 0; e < 8; e++) idx[e] = r[7 - e];
 }
 
-// Nibble form for BITS <= 4: nib[m], m = 0..3; the high nibble of byte b of
-// nib[m] is the index of element e = m, the low nibble that of e = m + 4, each
-// left-aligned in its nibble (index << (4 - BITS)).  Two butterfly stages.
-template <int BITS>
-AP_HD void planes_to_nibbles(const uint32_t (&q)[BITS], uint32_t (&nib)[4]) {
-    static_assert(BITS >= 1 && BITS <= 4, "index must fit a nibble");
-    // nibble bit i <- plane 3 - i; rows below 4 - BITS are zero
-    constexpr int LOW = 4 - BITS;
-    uint32_t r[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) r[i] = (i >= LOW) ? q[i >= LOW ? 3 - i : 0] : 0u;
-    swap_blocks<2, 0x33333333u, (0 < LOW), (2 < LOW)>(r[0], r[2]);
-    swap_blocks<2, 0x33333333u, (1 < LOW), (3 < LOW)>(r[1], r[3]);
-    constexpr bool Z02 = (0 < LOW) && (2 < LOW), Z13 = (1 < LOW) && (3 < LOW);
-    swap_blocks<1, 0x55555555u, Z02, Z13>(r[0], r[1]);
-    swap_blocks<1, 0x55555555u, Z02, Z13>(r[2], r[3]);
-    // r[u] nibble bit i = row i bit u of the nibble; element m sits at u = 3 - m.
-#pragma unroll
-    for (int m = 0; m < 4; m++) nib[m] = r[3 - m];
-}
-
-// Pair form (reference: dequant<3,true>, dequant<4,true>, dequant.cuh:13-30,
-// 56-67): byte b of pidx[m], m = 0..3, is
-//     ((index(e = m) << BITS) | index(e = m + 4)) << SHIFT.
-// BITS = 4, SHIFT = 0: the nibble form itself.  BITS = 3, SHIFT = 1: the high
-// nibble is built right-aligned and the low nibble left-aligned, so the two
-// 3-bit indices come out adjacent -- each butterfly row takes its low nibbles
-// from one plane and its high nibbles from the next.
-template <int BITS, int SHIFT>
-AP_HD void planes_to_pair_indices(const uint32_t (&q)[BITS], uint32_t (&pidx)[4]) {
-    static_assert((BITS == 4 && SHIFT == 0) || (BITS == 3 && SHIFT == 1), "supported pair forms");
-    if constexpr (BITS == 4) {
-        planes_to_nibbles<4>(q, pidx);
-    } else {
-        constexpr uint32_t LO = 0x0F0F0F0Fu;
-        uint32_t r[4];
-        r[3] = q[0] & LO;                    // low nibble bit 3 <- plane 0; high nibble bit 3 stays 0
-        r[2] = bit_select(LO, q[1], q[0]);   // low: plane 1, high: plane 0
-        r[1] = bit_select(LO, q[2], q[1]);   // low: plane 2, high: plane 1
-        r[0] = q[2] & ~LO;                   // low nibble bit 0 stays 0; high: plane 2
-        swap_blocks<2, 0x33333333u>(r[0], r[2]);
-        swap_blocks<2, 0x33333333u>(r[1], r[3]);
-        swap_blocks<1, 0x55555555u>(r[0], r[1]);
-        swap_blocks<1, 0x55555555u>(r[2], r[3]);
-#pragma unroll
-        for (int m = 0; m < 4; m++) pidx[m] = r[3 - m];
-    }
-}
-
 // Adjacent-pair form for BITS = 3, 4: apair[i], i = 0..3; byte b of apair[i] addresses the table entry
 // of the element PAIR (2i, 2i+1) of byte group 3 - b -- two elements that also share a dword of the
-// fp16 activations, so the activations need no rearranging (the form above pairs e with e + 4).
+// fp16 activations, so the activations need no rearranging (the reference's dequant<3,true> and
+// dequant<4,true>, dequant.cuh:13-30,56-67, pair element e with e + 4).
 // The byte holds the two indices bit-interleaved: with A = index(2i), B = index(2i+1) and A_k the bit
 // of weight 2^k,
 //     BITS = 4:  byte = A3 B3 A2 B2 A1 B1 A0 B0                       (entry number of a 256-entry table)

@@ -78,6 +78,31 @@ __device__ __forceinline__ uint32_t byte_add(uint32_t base, uint32_t v) {
     return r;
 }
 
+// A pointer into global memory that is the same in every lane, pinned to scalar registers: the compiler
+// then adds a lane's 32-bit byte offset in the load instruction itself (scalar base + vector offset)
+// instead of folding the base into 64-bit vector arithmetic per load.  The result carries the global
+// address space in its type, which the round trip through integers would otherwise lose.
+template <typename T>
+using global_ptr = __attribute__((address_space(1))) T *;
+
+template <typename T>
+__device__ __forceinline__ global_ptr<T> scalar_ptr(T *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (global_ptr<T>)(((uint64_t)hi << 32) | lo);
+}
+
+// Load of type V at byte offset `byte` (32 bits, per lane) from a scalar base.
+template <typename V, typename T>
+__device__ __forceinline__ V load_at(global_ptr<T> base, uint32_t byte) {
+    return *(global_ptr<const V>)((global_ptr<const char>)base + byte);
+}
+template <typename V, typename T>
+__device__ __forceinline__ V load_at_nt(global_ptr<T> base, uint32_t byte) {
+    return __builtin_nontemporal_load((global_ptr<const V>)((global_ptr<const char>)base + byte));
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
     const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true);

@@ -14,11 +14,11 @@ void launch_rows(const GemvGeometry &geo, const half_t *x, const GemvMembers &me
     const dim3 block(kWave, geo.S), grid(geo.grid);
     // smallest workgroup bound that holds S waves: leaves the most registers per lane
     if (geo.S <= 4)
-        gemv_kbit_kernel<BITS, M, WPL, R, 256><<<grid, block, 0, stream>>>(x, mem, K);
+        gemv_kbit_kernel<BITS, M, WPL, R, 256><<<grid, block, 0, stream>>>(x, mem, K, geo.S);
     else if (geo.S <= 8)
-        gemv_kbit_kernel<BITS, M, WPL, R, 512><<<grid, block, 0, stream>>>(x, mem, K);
+        gemv_kbit_kernel<BITS, M, WPL, R, 512><<<grid, block, 0, stream>>>(x, mem, K, geo.S);
     else
-        gemv_kbit_kernel<BITS, M, WPL, R, 1024><<<grid, block, 0, stream>>>(x, mem, K);
+        gemv_kbit_kernel<BITS, M, WPL, R, 1024><<<grid, block, 0, stream>>>(x, mem, K, geo.S);
 }
 
 template <int BITS, int M>
@@ -40,11 +40,11 @@ template <int BITS, int M>
 void launch_pair_m(const GemvGeometry &geo, const half_t *x, const GemvMembers &mem, int K, hipStream_t stream) {
     const dim3 block(kWave, geo.S), grid(geo.grid);
     if (geo.S <= 4)
-        gemv_kbit_kernel<BITS, M, 1, 2, 256, true><<<grid, block, 0, stream>>>(x, mem, K);
+        gemv_kbit_kernel<BITS, M, 1, 2, 256, true><<<grid, block, 0, stream>>>(x, mem, K, geo.S);
     else if (geo.S <= 8)
-        gemv_kbit_kernel<BITS, M, 1, 2, 512, true><<<grid, block, 0, stream>>>(x, mem, K);
+        gemv_kbit_kernel<BITS, M, 1, 2, 512, true><<<grid, block, 0, stream>>>(x, mem, K, geo.S);
     else
-        gemv_kbit_kernel<BITS, M, 1, 2, 1024, true><<<grid, block, 0, stream>>>(x, mem, K);
+        gemv_kbit_kernel<BITS, M, 1, 2, 1024, true><<<grid, block, 0, stream>>>(x, mem, K, geo.S);
 }
 
 }  // namespace

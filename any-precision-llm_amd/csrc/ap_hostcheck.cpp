@@ -21,36 +21,6 @@ int aph_planes_to_indices(const uint32_t *q, int bits, int shift, uint32_t *idx)
     return -1;
 }
 
-int aph_planes_to_pair_indices(const uint32_t *q, int bits, uint32_t *pidx) {
-    uint32_t out[4];
-    if (bits == 3) {
-        uint32_t qq[3] = {q[0], q[1], q[2]};
-        ap::planes_to_pair_indices<3, 1>(qq, out);
-    } else if (bits == 4) {
-        uint32_t qq[4] = {q[0], q[1], q[2], q[3]};
-        ap::planes_to_pair_indices<4, 0>(qq, out);
-    } else {
-        return -1;
-    }
-    for (int i = 0; i < 4; i++) pidx[i] = out[i];
-    return 0;
-}
-
-int aph_planes_to_nibbles(const uint32_t *q, int bits, uint32_t *nib) {
-    uint32_t out[4];
-#define AP_CASE(B)                                           \
-    if (bits == B) {                                         \
-        uint32_t qq[B];                                      \
-        for (int i = 0; i < B; i++) qq[i] = q[i];            \
-        ap::planes_to_nibbles<B>(qq, out);                   \
-        for (int i = 0; i < 4; i++) nib[i] = out[i];         \
-        return 0;                                            \
-    }
-    AP_CASE(1) AP_CASE(2) AP_CASE(3) AP_CASE(4)
-#undef AP_CASE
-    return -1;
-}
-
 int aph_planes_to_adjacent_pairs(const uint32_t *q, int bits, uint32_t *apair) {
     uint32_t out[4];
     if (bits == 3) {

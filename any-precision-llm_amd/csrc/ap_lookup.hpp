@@ -49,28 +49,39 @@ struct TableWords {
     u32x2 c;
 };
 
-// Issue the global loads of row `lut_row` (2^BITS fp16) for this lane.
+// Issue the global loads of row `lut_row` (2^BITS fp16) for this lane: a scalar row address plus the lane's
+// 32-bit byte offset.
 template <int BITS>
-__device__ __forceinline__ TableWords<BITS> lookup_table_fetch(const half_t *lut_row, int lane, const PairLane<BITS> &pl) {
+__device__ __forceinline__ TableWords<BITS> lookup_table_fetch(global_ptr<const half_t> lut_row, int lane, const PairLane<BITS> &pl) {
     TableWords<BITS> r;
     r.a = r.b = 0u;
     r.c = u32x2{0u, 0u};
-    const uint16_t *l16 = reinterpret_cast<const uint16_t *>(lut_row);
-    const uint32_t *l32 = reinterpret_cast<const uint32_t *>(lut_row);
     if constexpr (BITS == 3) {
-        r.a = l16[pl.first];
-        r.b = l16[pl.second];
+        r.a = load_at<uint16_t>(lut_row, pl.first * 2u);
+        r.b = load_at<uint16_t>(lut_row, pl.second * 2u);
     } else if constexpr (BITS == 4) {
-        r.a = l32[pl.first];
-        r.b = l32[pl.second];
+        r.a = load_at<uint32_t>(lut_row, pl.first * 4u);
+        r.b = load_at<uint32_t>(lut_row, pl.second * 4u);
     } else if constexpr (BITS == 8) {   // 512 B: 64 lanes x 8 B
-        r.c = reinterpret_cast<const u32x2 *>(lut_row)[lane];
+        r.c = load_at<u32x2>(lut_row, (uint32_t)lane * 8u);
     } else if constexpr (BITS == 7) {   // 256 B: 64 lanes x 4 B
-        r.a = l32[lane];
+        r.a = load_at<uint32_t>(lut_row, (uint32_t)lane * 4u);
     } else {                            // 64 / 128 B: first lanes x 4 B
-        if (lane < (1 << BITS) / 2) r.a = l32[lane];
+        if (lane < (1 << BITS) / 2) r.a = load_at<uint32_t>(lut_row, (uint32_t)lane * 4u);
     }
     return r;
+}
+template <int BITS>
+__device__ __forceinline__ TableWords<BITS> lookup_table_fetch(const half_t *lut_row, int lane, const PairLane<BITS> &pl) {
+    return lookup_table_fetch<BITS>(scalar_ptr(lut_row), lane, pl);
+}
+
+// A point the fetched words cannot be used before.  Put between the loads a kernel issues after the table
+// fetch and the staging: otherwise the compiler moves staging arithmetic (a shift of a fetched word) up to
+// the fetch, and the wave waits for its table before it has issued its plane loads.
+template <int BITS>
+__device__ __forceinline__ void lookup_table_arrive(TableWords<BITS> &r) {
+    asm volatile("" : "+v"(r.a), "+v"(r.b), "+v"(r.c));
 }
 
 // Write the fetched table into LDS in the form the lookups expect.
@@ -106,13 +117,16 @@ __device__ __forceinline__ void lds_only_barrier() {
 template <int M, int WPL>
 __device__ __forceinline__ void load_activations_plain(const half_t *__restrict__ x, int K, int wl,
                                                        uint32_t (&X)[M][WPL][4][4]) {
+    const global_ptr<const half_t> base = scalar_ptr(x);
 #pragma unroll
     for (int m = 0; m < M; m++)
 #pragma unroll
         for (int wi = 0; wi < WPL; wi++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const u32x4 v = *reinterpret_cast<const u32x4 *>(x + (size_t)m * K + group_base(wl + wi, j, K));
+                // uniform base + 32-bit byte offset of the lane (M * K * 2 < 2^32)
+                const uint32_t byte = ((uint32_t)m * (uint32_t)K + (uint32_t)group_base(wl + wi, j, K)) * 2u;
+                const u32x4 v = load_at<u32x4>(base, byte);
 #pragma unroll
                 for (int i = 0; i < 4; i++) X[m][wi][j][i] = v[i];
             }

@@ -38,19 +38,6 @@ def test_preshifted_indices(hostcheck, oracle, bits):
 
 
 @pytest.mark.parametrize("bits", [3, 4])
-def test_pair_indices(hostcheck, oracle, bits):
-    # byte = ((idx(e=m) << bits) | idx(e=m+4)) << shift; shift = 1 for 3 bits
-    shift = 1 if bits == 3 else 0
-    rng = np.random.default_rng(50 + bits)
-    for _ in range(300):
-        q = rng.integers(0, 2**32, size=bits, dtype=np.uint64).astype(np.uint32)
-        out = np.zeros(4, dtype=np.uint32)
-        assert hostcheck.aph_planes_to_pair_indices(ctypes.c_void_p(q.ctypes.data), bits,
-                                                    ctypes.c_void_p(out.ctypes.data)) == 0
-        assert np.array_equal(out, oracle.transpose_pair(q, bits) << np.uint32(shift))
-
-
-@pytest.mark.parametrize("bits", [3, 4])
 def test_adjacent_pair_indices(hostcheck, oracle, bits):
     """Byte b of apair[i] names the table entry of elements (2i, 2i+1) of byte group 3 - b: splitting it
     must give back the two indices the oracle's transpose holds for those elements (idx[e] byte b)."""
@@ -73,19 +60,6 @@ def test_adjacent_pair_indices(hostcheck, oracle, bits):
                 assert hostcheck.aph_adjacent_pair_split(bits, byte, ctypes.byref(first), ctypes.byref(second)) == 0
                 assert first.value == (int(want[2 * i]) >> (8 * b)) & 0xFF, (i, b)
                 assert second.value == (int(want[2 * i + 1]) >> (8 * b)) & 0xFF, (i, b)
-
-
-@pytest.mark.parametrize("bits", [1, 2, 3, 4])
-def test_nibble_indices(hostcheck, oracle, bits):
-    rng = np.random.default_rng(60 + bits)
-    for _ in range(300):
-        q = rng.integers(0, 2**32, size=bits, dtype=np.uint64).astype(np.uint32)
-        out = np.zeros(4, dtype=np.uint32)
-        assert hostcheck.aph_planes_to_nibbles(ctypes.c_void_p(q.ctypes.data), bits,
-                                               ctypes.c_void_p(out.ctypes.data)) == 0
-        s = oracle.transpose(q, bits)
-        want = ((s[:4] << np.uint32(4)) | s[4:]) << np.uint32(4 - bits)
-        assert np.array_equal(out, want)
 
 
 @pytest.mark.parametrize("K", [32, 64, 992, 1024, 1056, 4096, 11008, 14336])
