@@ -102,8 +102,22 @@ __device__ __forceinline__ void row_dot(const typename WordVec<WPL>::type (&q)[B
 // PAIR (R = 2 only): the two rows of a workgroup are row n of member 0 and row n of member 1 (two linears of
 // equal shape), and what is stored is silu(member 0) * member 1 -- the gate and up projections of a SwiGLU
 // MLP with their activation function, one output per row pair, nothing written in between.
+// Waves per SIMD the register allocator is asked to keep room for (1 = no request).  At 8 bits with two to
+// four activation rows the allocator, left alone, settles two or three registers above a step of the
+// occupancy table (83 where 80 fit six waves, 99 where 96 fit five) and a workgroup fewer fits the CU; the
+// request is what the registers a lane holds by design allow -- 16 per activation row for x, one per plane
+// and row, about 14 more -- out of 512 per SIMD lane in blocks of 8.  No instance spills with it; at fewer
+// bits the pair-table lookups in flight need more than the estimate, and the allocator does well alone.
+constexpr int gemv_waves_per_simd(int bits, int m, int wpl, int r) {
+    if (bits != 8 || wpl > 1 || m < 2 || m > 4) return 1;
+    const int need = 16 * m + r * bits + 14;
+    const int waves = 512 / ((need + 7) / 8 * 8);
+    return waves > 8 ? 8 : waves;
+}
+
 template <int BITS, int M, int WPL, int R, int THREADS, bool PAIR = false>
-__global__ __launch_bounds__(THREADS) void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K, int S) {
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(gemv_waves_per_simd(BITS, M, WPL, R))))
+void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K, int S) {
     static_assert(!PAIR || R == 2, "a pair is two rows");
     constexpr int NC = 1 << BITS;
     constexpr int MAXS = THREADS / kWave;

@@ -56,12 +56,15 @@ __global__ __launch_bounds__(THREADS) void gemvf_kbit_kernel(const half_t *__res
     const uint32_t *row_base = qweight + (size_t)(2 * pair) * W;
 #pragma unroll
     for (int p = 0; p < BITS; p++)  // streamed once: non-temporal, so x and the tables keep their cache lines
-        q[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(row_base + p * plane_stride + lane_off));
+        q[p] = load_at_nt<u32x2>(scalar_ptr(row_base + p * plane_stride), lane_off * (uint32_t)sizeof(uint32_t));
     uint32_t X[M][1][4][4];
     load_activations_plain<M, 1>(x, K, (int)w0, X);
 #pragma unroll
     for (int r = 0; r < 2; r++)
-        if (s == r % S) lookup_table_stage<BITS>(t[r], tables[r], lane);
+        if (s == r % S) {
+            lookup_table_arrive<BITS>(t[r]);  // staging arithmetic stays behind the plane and activation loads
+            lookup_table_stage<BITS>(t[r], tables[r], lane);
+        }
     if constexpr (kMulti) lds_only_barrier(); else __builtin_amdgcn_wave_barrier();
 
     uint32_t words[2][BITS];  // [row of the pair][plane]

@@ -38,7 +38,7 @@ __device__ __forceinline__ void load_pair(PairPlanes<BITS> &q, const uint32_t *_
                                           size_t plane_stride, uint32_t lane_off) {
 #pragma unroll
     for (int p = 0; p < BITS; p++)  // streamed once: non-temporal, so x and the tables keep their cache lines
-        q.v[p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row_base + p * plane_stride + lane_off));
+        q.v[p] = load_at_nt<u32x4>(scalar_ptr(row_base + p * plane_stride), lane_off * (uint32_t)sizeof(uint32_t));
 }
 
 // Grid: G workgroups of (64, S) threads, S = ceil(K / 4096) <= THREADS / 64; workgroup g takes the row
@@ -74,10 +74,13 @@ __global__ __launch_bounds__(THREADS) void gemvp_kbit_kernel(const half_t *__res
         for (int r = 0; r < 2; r++)
             if (s == r % S) t[r] = lookup_table_fetch<BITS>(lut + (size_t)(2 * pair + r) * NC, lane, pl);
     };
-    auto stage_tables = [&](const TableWords<BITS>(&t)[2], uint8_t(&slot)[2][LookupTable<BITS>::kBytes]) {
+    auto stage_tables = [&](TableWords<BITS>(&t)[2], uint8_t(&slot)[2][LookupTable<BITS>::kBytes]) {
 #pragma unroll
         for (int r = 0; r < 2; r++)
-            if (s == r % S) lookup_table_stage<BITS>(t[r], slot[r], lane);
+            if (s == r % S) {
+                lookup_table_arrive<BITS>(t[r]);  // staging arithmetic stays behind the loads issued since the fetch
+                lookup_table_stage<BITS>(t[r], slot[r], lane);
+            }
     };
 
     int pair = blockIdx.x;  // the grid never exceeds the number of pairs

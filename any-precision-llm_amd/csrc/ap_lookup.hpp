@@ -81,7 +81,9 @@ __device__ __forceinline__ TableWords<BITS> lookup_table_fetch(const half_t *lut
 // the fetch, and the wave waits for its table before it has issued its plane loads.
 template <int BITS>
 __device__ __forceinline__ void lookup_table_arrive(TableWords<BITS> &r) {
-    asm volatile("" : "+v"(r.a), "+v"(r.b), "+v"(r.c));
+    if constexpr (BITS <= 4) asm volatile("" : "+v"(r.a), "+v"(r.b));  // only the words this bit-width fetches
+    else if constexpr (BITS == 8) asm volatile("" : "+v"(r.c));
+    else asm volatile("" : "+v"(r.a));
 }
 
 // Write the fetched table into LDS in the form the lookups expect.
