@@ -222,6 +222,9 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
         }
     if (S > 1) lds_only_barrier(); else __builtin_amdgcn_wave_barrier();
 
+    // stores go through a pointer typed as global memory (the argument pointers left the statement above
+    // without an address space, and a store through them would be a flat one)
+    const global_ptr<half_t> out_g = (global_ptr<half_t>)reinterpret_cast<uint64_t>(out);
     float tot[R][M];
     static_for<R>([&](auto r_c) {
         constexpr int r = decltype(r_c)::value;
@@ -238,13 +241,13 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
         if (lane == kSumLane) {
             if constexpr (PAIR) {
 #pragma unroll
-                for (int m = 0; m < M; m++) out[(size_t)m * N + row0] = (half_t)swiglu(tot[0][m], tot[R - 1][m]);
+                for (int m = 0; m < M; m++) out_g[(size_t)m * N + row0] = (half_t)swiglu(tot[0][m], tot[R - 1][m]);
             } else {
 #pragma unroll
                 for (int r = 0; r < R; r++)
 #pragma unroll
                     for (int m = 0; m < M; m++)
-                        if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)tot[r][m];
+                        if (row0 + r < N) out_g[(size_t)m * N + row0 + r] = (half_t)tot[r][m];
             }
         }
     } else {
@@ -263,13 +266,17 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
                     g += partial[(ss * R) * M + tid];
                     u += partial[(ss * R + R - 1) * M + tid];
                 }
-                out[(size_t)tid * N + row0] = (half_t)swiglu(g, u);
+                out_g[(size_t)tid * N + row0] = (half_t)swiglu(g, u);
             }
         } else if (tid < R * M) {  // S >= 2 waves hold at least 128 threads >= R * M
             const int m = tid % M, r = tid / M;
             float v = 0.f;
-            for (int ss = 0; ss < S; ss++) v += partial[(ss * R + r) * M + m];
-            if (row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)v;
+            if (S == 2) {  // rows of up to 4096 elements: both partials in one LDS read instead of a loop of two
+                v = partial[r * M + m] + partial[(R + r) * M + m];
+            } else {
+                for (int ss = 0; ss < S; ss++) v += partial[(ss * R + r) * M + m];
+            }
+            if (row0 + r < N) out_g[(size_t)m * N + row0 + r] = (half_t)v;
         }
     }
 }
