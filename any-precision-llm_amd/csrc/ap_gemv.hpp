@@ -129,46 +129,37 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
     // arrives with the first clause of scalar loads (a branch per member costs a dependent scalar load
     // each) and the selects stay in scalar registers; no indexed access to the arguments.
     const int bid = blockIdx.x;
-    constexpr int NG = PAIR ? 2 : kGemvMaxGroup;
-    const uint32_t *m_q[NG];
-    const uint16_t *m_lut[NG];
-    uint16_t *m_out[NG];
-    int m_n[NG], m_end[NG], count = mem.count;
-#pragma unroll
-    for (int i = 0; i < NG; i++) {
-        m_q[i] = mem.qweight[i];
-        m_lut[i] = mem.lut[i];
-        m_out[i] = mem.out[i];
-        m_n[i] = mem.n[i];
-        m_end[i] = mem.wg_end[i];
-    }
-    // One empty statement that needs every argument in scalar registers: the compiler fetches them all
-    // with its first clause of scalar loads and waits once (left alone it loads each where it is first
-    // used, a dependent round trip to the scalar cache every time).
-    if constexpr (NG == 2)
-        asm volatile("" : "+s"(m_q[0]), "+s"(m_q[1]), "+s"(m_lut[0]), "+s"(m_lut[1]), "+s"(m_out[0]), "+s"(m_out[1]),
-                          "+s"(m_n[0]), "+s"(m_n[1]), "+s"(K), "+s"(S), "+s"(x));
+    // Member 0 (the only one of a plain call; with PAIR also member 1) and the scalars every workgroup
+    // needs, named in ONE empty statement that wants them in scalar registers: the compiler then fetches
+    // them with its first clause of scalar loads and waits once.  Left alone it loads each argument where
+    // it is first used, a dependent round trip to the scalar cache every time.
+    const uint32_t *q0 = mem.qweight[0], *q1 = mem.qweight[PAIR ? 1 : 0];
+    const uint16_t *lut0 = mem.lut[0], *lut1 = mem.lut[PAIR ? 1 : 0];
+    uint16_t *out0 = mem.out[0];
+    int n0 = mem.n[0], end0 = mem.wg_end[0], end1 = mem.wg_end[1], end2 = mem.wg_end[2], count = mem.count;
+    if constexpr (PAIR)
+        asm volatile("" : "+s"(q0), "+s"(q1), "+s"(lut0), "+s"(lut1), "+s"(out0), "+s"(n0), "+s"(K), "+s"(S), "+s"(x));
     else
-        asm volatile("" : "+s"(m_q[0]), "+s"(m_q[1]), "+s"(m_q[2]), "+s"(m_q[3]), "+s"(m_lut[0]), "+s"(m_lut[1]),
-                          "+s"(m_lut[2]), "+s"(m_lut[3]), "+s"(m_out[0]), "+s"(m_out[1]), "+s"(m_out[2]), "+s"(m_out[3]),
-                          "+s"(m_n[0]), "+s"(m_n[1]), "+s"(m_n[2]), "+s"(m_n[3]), "+s"(m_end[0]), "+s"(m_end[1]),
-                          "+s"(m_end[2]), "+s"(count), "+s"(K), "+s"(S), "+s"(x));
-    const uint32_t *__restrict__ qweight = m_q[0];
-    const half_t *__restrict__ lut = reinterpret_cast<const half_t *>(m_lut[0]);
-    half_t *__restrict__ out = reinterpret_cast<half_t *>(m_out[0]);
-    int N = m_n[0], wg0 = 0;
+        asm volatile("" : "+s"(q0), "+s"(lut0), "+s"(out0), "+s"(n0), "+s"(end0), "+s"(end1), "+s"(end2), "+s"(count),
+                          "+s"(K), "+s"(S), "+s"(x));
+    const uint32_t *__restrict__ qweight = q0;
+    const half_t *__restrict__ lut = reinterpret_cast<const half_t *>(lut0);
+    half_t *__restrict__ out = reinterpret_cast<half_t *>(out0);
+    int N = n0, wg0 = 0;
     if constexpr (!PAIR) {
-        if (count > 1) {  // a scalar branch: plain calls skip the selects
-            int g = 0;
-#pragma unroll
-            for (int i = 1; i < NG; i++) g = (i < count && bid >= m_end[i - 1]) ? i : g;  // wg_end ascends
-#pragma unroll
-            for (int i = 1; i < NG; i++) {
-                qweight = g == i ? m_q[i] : qweight;
-                lut = g == i ? reinterpret_cast<const half_t *>(m_lut[i]) : lut;
-                out = g == i ? reinterpret_cast<half_t *>(m_out[i]) : out;
-                N = g == i ? m_n[i] : N;
-                wg0 = g == i ? m_end[i - 1] : wg0;
+        if (count > 1) {
+            // a launch of several linears (a scalar branch; plain calls skip it): which member the workgroup
+            // belongs to, then that member's fields by index -- one more clause of scalar loads, cheaper than
+            // selecting each field among four
+            int g = bid >= end0 ? 1 : 0;  // wg_end ascends
+            g = (count > 2 && bid >= end1) ? 2 : g;
+            g = (count > 3 && bid >= end2) ? 3 : g;
+            if (g > 0) {
+                qweight = mem.qweight[g];
+                lut = reinterpret_cast<const half_t *>(mem.lut[g]);
+                out = reinterpret_cast<half_t *>(mem.out[g]);
+                N = mem.n[g];
+                wg0 = g == 1 ? end0 : (g == 2 ? end1 : end2);
             }
         }
     }
@@ -191,8 +182,8 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int n = PAIR ? row0 : min(row0 + r, N - 1);
-        plane_row[r] = reinterpret_cast<const char *>((PAIR ? m_q[r] : qweight) + (size_t)n * W);
-        table_row[r] = scalar_ptr((PAIR ? reinterpret_cast<const half_t *>(m_lut[r]) : lut) + (size_t)n * NC);
+        plane_row[r] = reinterpret_cast<const char *>((PAIR ? (r == 0 ? q0 : q1) : qweight) + (size_t)n * W);
+        table_row[r] = scalar_ptr((PAIR ? reinterpret_cast<const half_t *>(r == 0 ? lut0 : lut1) : lut) + (size_t)n * NC);
     }
 
     // Issue order matters: the tables first (tiny; staging them to LDS then overlaps the
@@ -200,11 +191,19 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
     // then the planes (HBM: the requests must go out at once), then the activations (L2
     // hits; issued before the planes they cost up to 1 us at 3-5 bits).  Rows past N (last
     // workgroup only) re-read row N-1 and are not stored.
+    // wave r % S fetches and stages the table of row r; r < 4, so up to three conditional subtractions
+    // instead of a division by a run-time S
+    auto stages = [&](int r) {
+        int owner = r;
+#pragma unroll
+        for (int i = 0; i < R - 1; i++) owner = owner >= S ? owner - S : owner;
+        return s == owner;
+    };
     const PairLane<BITS> pl = pair_lane<BITS>(lane);
     TableWords<BITS> t[R];
 #pragma unroll
     for (int r = 0; r < R; r++)
-        if (s == r % S) t[r] = lookup_table_fetch<BITS>(table_row[r], lane, pl);
+        if (stages(r)) t[r] = lookup_table_fetch<BITS>(table_row[r], lane, pl);
     wvec_t q[R][BITS];
 #pragma unroll
     for (int r = 0; r < R; r++)
@@ -216,7 +215,7 @@ void gemv_kbit_kernel(const half_t *__restrict__ x, const GemvMembers mem, int K
 
 #pragma unroll
     for (int r = 0; r < R; r++)
-        if (s == r % S) {
+        if (stages(r)) {
             lookup_table_arrive<BITS>(t[r]);
             lookup_table_stage<BITS>(t[r], tables[r], lane);
         }
