@@ -170,14 +170,19 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
 
 // One launch of the dequantiser over `count` linears (arguments already checked): fills the member table and sizes the grid.
 template <int BITS>
-void launch_dequant(const DequantMembers &mem, long long weights, hipStream_t stream) {
-    const long long items = mem.item_end[mem.count - 1];  // 64-word segments of all members
+void launch_dequant(const DequantMembers &mem, hipStream_t stream) {
+    const long long items = mem.items;  // 64-word segments of all members
     long long blocks = (items + kDequantWaves - 1) / kDequantWaves;
-    // Workgroups per CU the grid is capped at (the kernel strides over the rest): 32 measured best or within 1 % of
-    // best on every 7B..70B shape against 2..64; from about 128 M weights 64 is 5-6 % faster (28672 x 8192: a shorter
-    // tail).  The knob overrides when positive.
-    const int per_cu = knob(kDequantBlocksPerCu) > 0 ? knob(kDequantBlocksPerCu) : (weights >= (128LL << 20) ? 64 : 32);
-    const long long cap = (long long)cu_count() * per_cu;
+    // One item per wave (the hardware hands out workgroups as others retire) measured best or within 1-2 % of best
+    // from 15 workgroups per CU on, against caps of 3..64 per CU with waves striding over the rest (the seven linears of
+    // a Llama-2-7B layer in one launch: 85.5 / 107.5 us at 3 / 8 bits against 90 / 110 at 64 per CU).  A launch of 5..12
+    // workgroups per CU is resident all at once -- one burst of reads, then one of writes: capped at 5 per CU its
+    // waves take one or two items each, the second item's loads fly while the first one's stores drain, and it is 4-6 %
+    // faster (4096 x 4096: 9.3 -> 8.8 us at 3 bits, 12.4 -> 11.6 at 8).  The knob overrides when positive.
+    const long long cus = cu_count();
+    long long cap = blocks;
+    if (knob(kDequantBlocksPerCu) > 0) cap = cus * knob(kDequantBlocksPerCu);
+    else if (blocks > 5 * cus && blocks <= 12 * cus) cap = 5 * cus;
     if (blocks > cap) blocks = cap;
     dequant_kbit_kernel<BITS><<<dim3((unsigned)blocks), dim3(kDequantWaves * kWave), 0, stream>>>(mem);
 }
@@ -340,33 +345,35 @@ int ap_dequant_kbit_group(int count, const uint32_t *const *qweight, const uint1
     if (!qweight || !lut || !out || !N || !K) return AP_ENULL;
     if (count < 1 || count > kDequantMaxGroup) return AP_ELIMIT;
     DequantMembers mem = {};
-    long long items = 0, weights = 0;
+    long long items = 0;
     for (int g = 0; g < count; g++) {
         if (!qweight[g] || !lut[g] || !out[g]) return AP_ENULL;
         const int rc = check_common(N[g], K[g], w_bits);
         if (rc != AP_OK) return rc;
         if (!aligned16(qweight[g]) || !aligned16(lut[g]) || !aligned16(out[g])) return AP_EALIGN;
         const long long segs = (long long)N[g] * (((K[g] >> 5) + kWave - 1) / kWave);
-        if (segs > 0x7fffffffLL) return AP_ELIMIT;
         items += segs;
-        weights += (long long)N[g] * K[g];
+        if (items > 0x7fffffffLL) return AP_ELIMIT;  // the kernel numbers the segments of a launch in 32 bits
+        const unsigned long long per_row = (unsigned long long)(((K[g] >> 5) + kWave - 1) / kWave);
+        mem.seg_magic[g] = per_row == 1 ? 0xffffffffu : (uint32_t)((1ULL << 32) / per_row);
         mem.qweight[g] = qweight[g];
         mem.lut[g] = lut[g];
         mem.out[g] = out[g];
         mem.N[g] = N[g];
         mem.K[g] = K[g];
-        mem.item_end[g] = items;
+        mem.item_end[g] = (int)items;
     }
+    mem.items = (int)items;
     mem.count = count;
     hipStream_t st = static_cast<hipStream_t>(stream);
     drain_stale_error();
     switch (w_bits) {
-        case 3: launch_dequant<3>(mem, weights, st); break;
-        case 4: launch_dequant<4>(mem, weights, st); break;
-        case 5: launch_dequant<5>(mem, weights, st); break;
-        case 6: launch_dequant<6>(mem, weights, st); break;
-        case 7: launch_dequant<7>(mem, weights, st); break;
-        default: launch_dequant<8>(mem, weights, st); break;
+        case 3: launch_dequant<3>(mem, st); break;
+        case 4: launch_dequant<4>(mem, st); break;
+        case 5: launch_dequant<5>(mem, st); break;
+        case 6: launch_dequant<6>(mem, st); break;
+        case 7: launch_dequant<7>(mem, st); break;
+        default: launch_dequant<8>(mem, st); break;
     }
     return launch_status();
 }

@@ -102,6 +102,10 @@ template <typename V, typename T>
 __device__ __forceinline__ V load_at_nt(global_ptr<T> base, uint32_t byte) {
     return __builtin_nontemporal_load((global_ptr<const V>)((global_ptr<const char>)base + byte));
 }
+template <typename V, typename T>
+__device__ __forceinline__ void store_at_nt(global_ptr<T> base, uint32_t byte, const V &v) {
+    __builtin_nontemporal_store(v, (global_ptr<V>)((global_ptr<char>)base + byte));
+}
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_add(float v) {
@@ -136,18 +140,30 @@ struct LutRegs {
 };
 
 template <int BITS>
-__device__ __forceinline__ LutRegs<BITS> lut_fetch(const half_t *lut_row, int lane) {
+__device__ __forceinline__ LutRegs<BITS> lut_fetch(global_ptr<const half_t> lut_row, int lane) {
     LutRegs<BITS> r;
     r.v = u32x2{0u, 0u};
     constexpr int dwords = (1 << BITS) / 2;          // table size in dwords
     if constexpr (dwords >= 128) {                   // 8 bits: 64 lanes x 8 B
-        r.v = reinterpret_cast<const u32x2 *>(lut_row)[lane];
+        r.v = load_at<u32x2>(lut_row, (uint32_t)lane * 8u);
     } else if constexpr (dwords == 64) {             // 7 bits: 64 lanes x 4 B
-        r.v.x = reinterpret_cast<const uint32_t *>(lut_row)[lane];
+        r.v.x = load_at<uint32_t>(lut_row, (uint32_t)lane * 4u);
     } else {                                         // <= 6 bits: first `dwords` lanes
-        if (lane < dwords) r.v.x = reinterpret_cast<const uint32_t *>(lut_row)[lane];
+        if (lane < dwords) r.v.x = load_at<uint32_t>(lut_row, (uint32_t)lane * 4u);
     }
     return r;
+}
+template <int BITS>
+__device__ __forceinline__ LutRegs<BITS> lut_fetch(const half_t *lut_row, int lane) {
+    return lut_fetch<BITS>(scalar_ptr(lut_row), lane);
+}
+
+// A point the fetched words cannot be used before: put between the loads a kernel issues after the table
+// fetch and the staging, so that no staging work is moved up to the fetch (and the wave made to wait for its
+// table before its other loads have left).
+template <int BITS>
+__device__ __forceinline__ void lut_arrive(LutRegs<BITS> &r) {
+    if constexpr (BITS == 8) asm volatile("" : "+v"(r.v)); else asm volatile("" : "+v"(r.v.x));
 }
 
 template <int BITS>
