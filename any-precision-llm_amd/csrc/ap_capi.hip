@@ -481,8 +481,8 @@ bool gemmt_pays(int M, int N, int K, int w_bits) {
 // Launch of the fused dequant -> MFMA kernel (arguments already checked).
 int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, uint16_t *out, int M, int N, int K,
              int w_bits, hipStream_t st) {
-    // the kernel addresses the activations with 32-bit byte offsets
-    if ((long long)M * K * 2 > 0xffffffffLL) return AP_ELIMIT;
+    // the kernels address the activations, and a row inside a plane, with 32-bit byte offsets
+    if ((long long)M * K * 2 > 0xffffffffLL || (long long)N * (K >> 5) * 4 > 0xffffffffLL) return AP_ELIMIT;
     {
         GemmwGeometry wgeo;
         const int mode = knob(kGemmWalk);

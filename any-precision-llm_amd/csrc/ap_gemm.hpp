@@ -63,7 +63,7 @@ __device__ __forceinline__ void transpose_rows4(uint32_t (&r)[4]) {
 template <int BITS, int MB, bool VEC4, int MP, int RB>
 __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
-    half_t *__restrict__ out, int M, int N, int K) {
+    half_t *__restrict__ out, int M, int N, int K, int KS, uint32_t ks_magic) {
     constexpr int NC = 1 << BITS;
     constexpr int WPS = VEC4 ? 4 : 1;             // words per lane and step
     constexpr int ROWS = kGemmRows * RB;    // weight rows per workgroup
@@ -81,20 +81,30 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     __shared__ u32x4 xs[kGemmMaxSplit][XS];
     static_assert(MP == 0 || (MP >= 8 && MP <= 16 * MB && (MP & (MP - 1)) == 0), "");
 
+    // every argument in scalar registers by one clause of scalar loads and one wait (the compiler alone loads
+    // an argument where it is first used: a dependent round trip to the scalar cache each)
+    asm volatile("" : "+s"(x), "+s"(qweight), "+s"(lut), "+s"(out), "+s"(M), "+s"(N), "+s"(K), "+s"(KS), "+s"(ks_magic));
     const int lane = threadIdx.x;
-    const int ks = __builtin_amdgcn_readfirstlane(threadIdx.y), KS = blockDim.y;
+    const int ks = __builtin_amdgcn_readfirstlane(threadIdx.y);  // KS = blockDim.y, passed as an argument
     const int col = lane & 15, grp = lane >> 4;
     const int W = K >> 5;
-    const size_t plane_stride = (size_t)N * W;
+    const size_t plane_bytes = (size_t)N * W * sizeof(uint32_t);  // below 2^32 (the host checks)
     const int n0 = blockIdx.x * ROWS;
 
-    // this wave's range of steps (4 * WPS words of every row per step)
+    // this wave's range of steps (4 * WPS words of every row per step): steps * ks / KS by a multiplication
+    // with ks_magic = ceil(2^32 / KS) from the host, exact for steps * (ks + 1) < 2^29 (KS <= 8, K < 2^33)
     const int steps = (W + 4 * WPS - 1) / (4 * WPS);
-    const int s_begin = steps * ks / KS, s_end = steps * (ks + 1) / KS;  // steps < 2^26, KS <= 8: no overflow
+    auto over_ks = [&](int n) { return KS == 1 ? n : (int)__umulhi((uint32_t)n, ks_magic); };
+    const int s_begin = over_ks(steps * ks), s_end = over_ks(steps * (ks + 1));
 
-    const uint32_t *wrow[RB];  // rows past N repeat row N-1 and are not stored
+    // byte offset of this lane's row inside a plane (rows past N repeat row N-1 and are not stored); a plane
+    // word is loaded from the scalar plane base plus this offset plus the word's
+    const global_ptr<const char> qbytes = scalar_ptr(reinterpret_cast<const char *>(qweight));
+    const global_ptr<const half_t> xg = scalar_ptr(x);
+    uint32_t row_off[RB];
 #pragma unroll
-    for (int rb = 0; rb < RB; rb++) wrow[rb] = qweight + (size_t)min(n0 + rb * kGemmRows + col, N - 1) * W;
+    for (int rb = 0; rb < RB; rb++)
+        row_off[rb] = (uint32_t)min(n0 + rb * kGemmRows + col, N - 1) * (uint32_t)W * (uint32_t)sizeof(uint32_t);
     // q[rb][p][i]: row block rb, plane p, i-th word of this lane for the step
     auto fetch = [&](int step, uint32_t(&q)[RB][BITS][WPS]) {
         if constexpr (VEC4) {
@@ -105,8 +115,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
             for (int rb = 0; rb < RB; rb++)
 #pragma unroll
                 for (int p = 0; p < BITS; p++) {
-                    const u32x4 v =
-                        __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(wrow[rb] + p * plane_stride + w));
+                    const u32x4 v = load_at_nt<u32x4>(scalar_ptr(qbytes + p * plane_bytes), row_off[rb] + (uint32_t)w * 4u);
 #pragma unroll
                     for (int i = 0; i < 4; i++) q[rb][p][i] = v[i];
                 }
@@ -116,7 +125,8 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 #pragma unroll
             for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-                for (int p = 0; p < BITS; p++) q[rb][p][0] = wrow[rb][p * plane_stride + w];
+                for (int p = 0; p < BITS; p++)
+                    q[rb][p][0] = load_at<uint32_t>(scalar_ptr(qbytes + p * plane_bytes), row_off[rb] + (uint32_t)w * 4u);
         }
     };
 
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
             lookup_table_stage<BITS>(lookup_table_fetch<BITS>(lut + (size_t)min(n0 + r, N - 1) * NC, lane, pl), &tables[r][0], lane);
     } else {
         const int nthr = KS * kWave;
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(lut);
+        const global_ptr<const u32x4> src = (global_ptr<const u32x4>)reinterpret_cast<uint64_t>(lut);
         u32x4 *dst = reinterpret_cast<u32x4 *>(&tables[0][0]);
         const long long first = (long long)n0 * (NC / 8), last = (long long)N * (NC / 8) - 1;
         for (int i = ks * kWave + lane; i < TQ; i += nthr) dst[i] = src[min(first + i, last)];
@@ -207,7 +217,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
                 const uint32_t koff = kb[t / 4] + (uint32_t)(t % 4) * jstride[t / 4];
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
-                    a[t][mb] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(x) + (size_t)(xoff[mb] + koff));
+                    a[t][mb] = load_at<half8_t>(xg, xoff[mb] + koff);
             }
         };
         // ---- staged path (MP > 0): lane = (row r + 4 i, byte group sj, octet sg of the run)
@@ -223,7 +233,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 #pragma unroll
                 for (int i = 0; i < NL; i++) {
                     const uint32_t roff = (uint32_t)min(sr + 4 * i, M - 1) * (uint32_t)K * 2u;
-                    xr[i] = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const char *>(x) + (size_t)(roff + koff));
+                    xr[i] = load_at<u32x4>(xg, roff + koff);
                 }
             }
         };
@@ -342,6 +352,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 
     // Combine the K-split partial tiles in wave order (also with one wave: it keeps the
     // accumulator indices static).  D[i][j]: lane l holds rows i = 4 (l / 16) + v, column l % 16.
+    const global_ptr<half_t> out_g = (global_ptr<half_t>)reinterpret_cast<uint64_t>(out);  // a global store, not a flat one
     float *mine = reinterpret_cast<float *>(&xs[ks][0]);
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
@@ -355,7 +366,7 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
         float sum = 0.f;
         for (int kk = 0; kk < KS; kk++) sum += reinterpret_cast<const float *>(&xs[kk][0])[t * kWave + lane];
         const int m = mb * 16 + 4 * grp + v, n = n0 + rb * kGemmRows + col;
-        if (m < M && n < N) out[(size_t)m * N + n] = (half_t)sum;
+        if (m < M && n < N) out_g[(size_t)m * N + n] = (half_t)sum;
     }
 }
 

@@ -15,20 +15,22 @@ void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qwe
     half_t *oh = reinterpret_cast<half_t *>(out);
     const dim3 block(kWave, geo.ks), grid(geo.grid);
     const bool vec4 = ((K >> 5) & 3) == 0;  // whole 16-byte quads of words per row
+    // ceil(2^32 / ks): the kernel divides its step counts by ks with one multiplication (unused when ks == 1)
+    const uint32_t ks_magic = geo.ks > 1 ? (uint32_t)(((1ULL << 32) + (unsigned)geo.ks - 1) / (unsigned)geo.ks) : 0u;
     // Two row blocks (17..32 activation rows) stage the activations through LDS (measured
     // 10-17 % faster at every bit-width); one row block is as fast or faster straight from
     // global memory, and beyond two the staging region would crowd out the second workgroup
     // of a CU.
 #define AP_GEMM_LAUNCH(MBV, MPV)                                                                                     \
     do {                                                                                                             \
-        if (vec4) gemm_kbit_kernel<BITS, MBV, true, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);   \
-        else gemm_kbit_kernel<BITS, MBV, false, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);       \
+        if (vec4) gemm_kbit_kernel<BITS, MBV, true, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);   \
+        else gemm_kbit_kernel<BITS, MBV, false, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);       \
     } while (0)
 #define AP_GEMM_CASE(MBV) \
     case MBV: AP_GEMM_LAUNCH(MBV, 0); break;
     if (geo.rb == 2) {  // chosen by the caller only with vec4 and at most two activation row blocks
-        if (geo.mb == 1) gemm_kbit_kernel<BITS, 1, true, 0, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
-        else gemm_kbit_kernel<BITS, 2, true, 32, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K);
+        if (geo.mb == 1) gemm_kbit_kernel<BITS, 1, true, 0, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);
+        else gemm_kbit_kernel<BITS, 2, true, 32, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);
         return;
     }
     switch (geo.mb) {
