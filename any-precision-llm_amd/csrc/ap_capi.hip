@@ -354,8 +354,7 @@ int ap_dequant_kbit_group(int count, const uint32_t *const *qweight, const uint1
         const long long segs = (long long)N[g] * (((K[g] >> 5) + kWave - 1) / kWave);
         items += segs;
         if (items > 0x7fffffffLL) return AP_ELIMIT;  // the kernel numbers the segments of a launch in 32 bits
-        const unsigned long long per_row = (unsigned long long)(((K[g] >> 5) + kWave - 1) / kWave);
-        mem.seg_magic[g] = per_row == 1 ? 0xffffffffu : (uint32_t)((1ULL << 32) / per_row);
+        mem.seg_magic[g] = reciprocal_floor((uint32_t)(((K[g] >> 5) + kWave - 1) / kWave));
         mem.qweight[g] = qweight[g];
         mem.lut[g] = lut[g];
         mem.out[g] = out[g];
@@ -616,6 +615,7 @@ int run_gemv4(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, u
     Gemv4Geometry geo;
     if (M > 8) return AP_EBATCH;
     const int W = K >> 5;
+    if ((long long)N * W * 4 > 0xffffffffLL) return AP_ELIMIT;  // the kernel addresses a row inside a plane with 32 bits
     if (M > 4) {
         // two groups of four activation rows: four row quads per workgroup, one word group per wave
         geo.mg = 2;

@@ -15,6 +15,7 @@
 #pragma once
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
+#include "ap_reciprocal.hpp"
 
 namespace ap {
 
@@ -23,7 +24,7 @@ constexpr int kDequantMaxGroup = 8;  // linears one launch can serve (any shapes
 
 // The linears of one launch, passed by value as kernel arguments.  The 64-word segments of all members are
 // numbered through: member g owns items [item_end[g-1], item_end[g]); `items` is the total (below 2^31, the host
-// checks).  seg_magic[g] = floor(2^32 / S_g), S_g the segments of a row of member g (2^32 - 1 for S_g = 1): the
+// checks).  seg_magic[g] = reciprocal_floor(S_g), S_g the segments of a row of member g (ap_reciprocal.hpp): the
 // kernel divides an item number by S_g with one multiply and one correction step instead of a division.
 struct DequantMembers {
     const uint32_t *qweight[kDequantMaxGroup];
@@ -108,10 +109,8 @@ __global__ __launch_bounds__(kDequantWaves * kWave) void dequant_kbit_kernel(con
         it.W = K >> 5;
         const uint32_t S = (uint32_t)(it.W + kWave - 1) / kWave;  // segments per row
         const uint32_t local = (uint32_t)(item - first);
-        uint32_t row = __umulhi(local, magic), seg = local - row * S;  // row is the quotient or one below it
-        const uint32_t fix = (S - 1u - seg) >> 31;  // 1 when seg >= S (both below 2^31)
-        row += fix;
-        seg -= S & (0u - fix);
+        uint32_t row, seg;
+        divmod_by_reciprocal(local, S, magic, row, seg);
         it.seg = (int)seg;
         it.plane_bytes = (size_t)N * it.W * sizeof(uint32_t);
         it.planes = scalar_ptr(reinterpret_cast<const char *>(qw + (size_t)row * it.W));

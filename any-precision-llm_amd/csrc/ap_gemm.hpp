@@ -34,6 +34,7 @@
 #include "ap_device.hpp"
 #include "ap_gemm_launch.hpp"
 #include "ap_lookup.hpp"
+#include "ap_reciprocal.hpp"
 
 namespace ap {
 
@@ -92,9 +93,10 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const int n0 = blockIdx.x * ROWS;
 
     // this wave's range of steps (4 * WPS words of every row per step): steps * ks / KS by a multiplication
-    // with ks_magic = ceil(2^32 / KS) from the host, exact for steps * (ks + 1) < 2^29 (KS <= 8, K < 2^33)
+    // with ks_magic = reciprocal_ceil(KS) from the host (ap_reciprocal.hpp), exact for steps * (ks + 1) < 2^29
+    // (KS <= 8, K < 2^33)
     const int steps = (W + 4 * WPS - 1) / (4 * WPS);
-    auto over_ks = [&](int n) { return KS == 1 ? n : (int)__umulhi((uint32_t)n, ks_magic); };
+    auto over_ks = [&](int n) { return (int)div_by_reciprocal_ceil((uint32_t)n, (uint32_t)KS, ks_magic); };
     const int s_begin = over_ks(steps * ks), s_end = over_ks(steps * (ks + 1));
 
     // byte offset of this lane's row inside a plane (rows past N repeat row N-1 and are not stored); a plane

@@ -15,12 +15,7 @@ void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qwe
     half_t *oh = reinterpret_cast<half_t *>(out);
     const dim3 block(kWave, geo.ks), grid(geo.grid);
     const bool vec4 = ((K >> 5) & 3) == 0;  // whole 16-byte quads of words per row
-    // ceil(2^32 / ks): the kernel divides its step counts by ks with one multiplication (unused when ks == 1)
-    const uint32_t ks_magic = geo.ks > 1 ? (uint32_t)(((1ULL << 32) + (unsigned)geo.ks - 1) / (unsigned)geo.ks) : 0u;
-    // Two row blocks (17..32 activation rows) stage the activations through LDS (measured
-    // 10-17 % faster at every bit-width); one row block is as fast or faster straight from
-    // global memory, and beyond two the staging region would crowd out the second workgroup
-    // of a CU.
+    const uint32_t ks_magic = reciprocal_ceil((uint32_t)geo.ks);  // the kernel divides its step counts by ks with one multiplication
 #define AP_GEMM_LAUNCH(MBV, MPV)                                                                                     \
     do {                                                                                                             \
         if (vec4) gemm_kbit_kernel<BITS, MBV, true, MPV, 1><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);   \

@@ -59,8 +59,11 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     const int s = __builtin_amdgcn_readfirstlane(threadIdx.y), S = blockDim.y;
     const int qi = lane & 3, wb = lane >> 2;
     const int W = K >> 5;
-    const size_t plane_stride = (size_t)N * W;
+    const size_t plane_bytes = (size_t)N * W * sizeof(uint32_t);  // below 2^32 (the host checks)
     const int row0 = blockIdx.x * ROWS;
+    // loads are a scalar base plus a 32-bit byte offset per lane (no 64-bit vector arithmetic per load)
+    const global_ptr<const char> qbytes = scalar_ptr(reinterpret_cast<const char *>(qweight));
+    const global_ptr<const half_t> xg = scalar_ptr(x);
 
     // Load order as in the dot-product kernel: tables, planes (non-temporal: streamed once),
     // activations.
@@ -88,24 +91,24 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
 #pragma unroll
     for (int rq = 0; rq < RQ; rq++) {
         // rows past N repeat row N-1 and are not stored
-        const uint32_t *wrow = qweight + (size_t)min(row0 + 4 * rq + lrow, N - 1) * W;
+        const uint32_t row_words = (uint32_t)min(row0 + 4 * rq + lrow, N - 1) * (uint32_t)W;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const int w = min((s * G + g) * 16 + lword, W - 1);
+            const uint32_t byte = (row_words + (uint32_t)min((s * G + g) * 16 + lword, W - 1)) * (uint32_t)sizeof(uint32_t);
 #pragma unroll
-            for (int p = 0; p < BITS; p++) q[rq][g][p] = __builtin_nontemporal_load(wrow + p * plane_stride + w);
+            for (int p = 0; p < BITS; p++) q[rq][g][p] = load_at_nt<uint32_t>(scalar_ptr(qbytes + p * plane_bytes), byte);
         }
     }
     // X[mg][g][j]: the eight activations of byte group j of this lane's word, row 4 mg + qi
     u32x4 X[MG][G][4];
 #pragma unroll
     for (int mg = 0; mg < MG; mg++) {
-        const half_t *xrow = x + (size_t)min(mg * 4 + qi, M - 1) * K;
+        const uint32_t xrow = (uint32_t)min(mg * 4 + qi, M - 1) * (uint32_t)K;  // M * K * 2 < 2^32 (M <= 8)
 #pragma unroll
         for (int g = 0; g < G; g++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                X[mg][g][j] = *reinterpret_cast<const u32x4 *>(xrow + group_base(wl[g], j, K));
+                X[mg][g][j] = load_at<u32x4>(xg, (xrow + (uint32_t)group_base(wl[g], j, K)) * (uint32_t)sizeof(half_t));
     }
     // words past the row end (last wave of a row only): all four lanes of their block are past it,
     // so zero activations silence the whole block

@@ -2,6 +2,7 @@
 // Compiled with g++ into libanyprec_hostcheck.so; exports the in-lane plane ->
 // index transposes and the layout address helpers exactly as the kernels use them.
 #include "ap_bitplane.hpp"
+#include "ap_reciprocal.hpp"
 
 extern "C" {
 
@@ -45,5 +46,19 @@ int aph_adjacent_pair_split(int bits, uint32_t byte, uint32_t *first, uint32_t *
 
 int aph_chunk_words(int w, int K) { return ap::chunk_words(w, K); }
 int aph_group_base(int w, int j, int K) { return ap::group_base(w, j, K); }
+
+// n / d and n % d through the host-side reciprocal, as the dequantiser numbers its segments (n < 2^31)
+int aph_divmod_by_reciprocal(uint32_t n, uint32_t d, uint32_t *q, uint32_t *r) {
+    if (d < 1 || d >= (1u << 31) || n >= (1u << 31)) return -1;
+    ap::divmod_by_reciprocal(n, d, ap::reciprocal_floor(d), *q, *r);
+    return 0;
+}
+
+// n / d as the K-split GEMM splits its steps over d waves (n * d < 2^32)
+int aph_div_by_reciprocal_ceil(uint32_t n, uint32_t d, uint32_t *q) {
+    if (d < 1 || (unsigned long long)n * d >= (1ull << 32)) return -1;
+    *q = ap::div_by_reciprocal_ceil(n, d, ap::reciprocal_ceil(d));
+    return 0;
+}
 
 }  // extern "C"

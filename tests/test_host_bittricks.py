@@ -95,3 +95,33 @@ def test_group_base_matches_packer(hostcheck, oracle):
         expect = np.zeros(W, dtype=np.uint32)
         expect[w] = np.uint32(1 << bit)
         assert np.array_equal(qw, expect)
+
+
+def test_division_by_host_reciprocal_is_exact(hostcheck):
+    """The kernels divide by a run-time divisor with a reciprocal from the launch code (ap_reciprocal.hpp).
+    Against Python's integer division: every divisor up to 600 with numerators around every multiple boundary and
+    at the top of the range, and random pairs over the whole range the kernels allow."""
+    q, r = ctypes.c_uint32(), ctypes.c_uint32()
+    rng = np.random.default_rng(7)
+    top = 2**31 - 1
+    for d in list(range(1, 601)) + [1023, 1024, 4097, 65535, 65536, 2**20 + 1, 2**30, top]:
+        ns = {0, 1, d - 1, d, d + 1, top, top - 1, (top // d) * d, max((top // d) * d - 1, 0)}
+        ns |= {int(k) * d + o for k in rng.integers(0, max(top // d, 1), size=6) for o in (-1, 0, 1)}
+        for n in ns:
+            if 0 <= n <= top:
+                assert hostcheck.aph_divmod_by_reciprocal(n, d, ctypes.byref(q), ctypes.byref(r)) == 0
+                assert (q.value, r.value) == divmod(n, d), (n, d)
+    for n, d in zip(rng.integers(0, 2**31, size=20000), rng.integers(1, 2**31, size=20000)):
+        assert hostcheck.aph_divmod_by_reciprocal(int(n), int(d), ctypes.byref(q), ctypes.byref(r)) == 0
+        assert (q.value, r.value) == divmod(int(n), int(d)), (n, d)
+    # the K-split form: no correction step, exact while n * d < 2^32
+    for d in range(1, 17):
+        lim = 2**32 // d
+        ns = {0, 1, d - 1, d, lim - 1, lim - 2, (lim - 1) // d * d, (lim - 1) // d * d - 1}
+        ns |= {int(v) for v in rng.integers(0, lim, size=4000)}
+        for n in ns:
+            if 0 <= n < lim:
+                assert hostcheck.aph_div_by_reciprocal_ceil(n, d, ctypes.byref(q)) == 0
+                assert q.value == n // d, (n, d)
+    assert hostcheck.aph_div_by_reciprocal_ceil(2**31, 2, ctypes.byref(q)) == -1   # outside the exact range: refused
+    assert hostcheck.aph_divmod_by_reciprocal(2**31, 3, ctypes.byref(q), ctypes.byref(r)) == -1
