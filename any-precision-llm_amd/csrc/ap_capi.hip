@@ -89,10 +89,13 @@ int check_common(int N, int K, int w_bits) {
 //          needs two word groups per wave there and doubles its time from 4 bits on (5120 x 13824, M = 3, 4 bits:
 //          28.9 us against 18.5) --, but 10-35 % SLOWER on rows of 11008 elements (workgroups of 6 waves: two of them
 //          fit a CU at the four-row kernel's register count, three at the two-row kernel's), which keep their routes.
-bool long_rows_want_four(int M, int K) {
+// Swept again after the kernels' prologues were trimmed: at M = 2 and up to 4 bits rows of 7-8 waves (13824, 14336,
+// 16384 elements) are 7-13 % faster with four rows than with the row-streaming kernel that served them (4096 x 14336,
+// 3 bits: 12.1 -> 10.6 us); rows of 14 waves (28672) are 22 % slower and stay with it.
+bool long_rows_want_four(int M, int K, int w_bits) {
     const int W = K >> 5, S = (W + kWave - 1) / kWave;
     if (M < 2 || M > 4 || K < 8192 || S > kGemvMaxSeg) return false;
-    return M == 2 ? S <= 6 : (S <= 4 || S >= 7);
+    return M == 2 ? (S <= 6 || (S <= 8 && w_bits <= 4)) : (S <= 4 || S >= 7);
 }
 
 // Four activation rows at 6-8 bits on rows of 4097..8191 elements (5120 x 5120, 13824 x 5120): four weight rows per
@@ -127,6 +130,10 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
     // on); 4096 x 4096 (8192 waves) keeps one.
     const long long tw = target_waves > 0 ? ((w_bits <= 4 || (M == 2 && count == 1)) ? (long long)target_waves * 3 / 4 : target_waves) : 1;
     int R = force_rows > 0 ? force_rows : (rows * S >= tw ? 2 : 1);
+    // Two activation rows at up to 4 bits: two weight rows from 4096 waves on (4096 x 4096, 8192 waves: 7-9 % faster,
+    // 3 bits 5.5 -> 5.0 us; 1024 x 4096, 2048 waves, is 6 % slower with two and keeps one; from 5 bits on 4096 x 4096
+    // is 3-11 % slower with two).
+    if (force_rows <= 0 && M == 2 && count == 1 && w_bits <= 4 && rows * S >= 4096) R = 2;
     R = (R >= 2 || M > 2) ? 2 : 1;
     // Four rows per workgroup (one activation row, one word per lane): the activations a wave holds then serve
     // four rows, which halves their traffic through the L1 once more, at the price of half the waves.  Measured
@@ -147,7 +154,7 @@ int gemv_geometry(int M, const int *n, int count, int K, int w_bits, GemvGeometr
         const long long waves = rows * S;
         const bool pays = M == 1 ? (count == 1 ? waves >= 28000 && (w_bits <= 4 || (K >= 8192 && waves >= 32768))
                                                : waves >= 20000 && w_bits <= 4)
-                                 : long_rows_want_four(M, K) || mid_rows_want_four(M, K, w_bits) ||
+                                 : long_rows_want_four(M, K, w_bits) || mid_rows_want_four(M, K, w_bits) ||
                                    (count > 1 && (M >= 3 || w_bits <= 4));
         if (force_rows == 4 || (force_rows <= 0 && pays)) R = 4;
     }
@@ -695,22 +702,24 @@ int few_rows_route(const RouteQuery &q) {
     // 5-9 % on 1024 x 4096 at 3-4 rows and up to 4 bits
     if (single(q) && fine_ok && q.lo <= 2048 && ((K >= 8192 && M >= 2) || (M >= 3 && b <= 4))) return AP_ROUTE_FINE;
     // long rows at 2..4 rows: gemv_kbit_kernel with four rows per workgroup (gemv_geometry shapes it so) wherever
-    // long_rows_want_four says -- except M = 3 on rows of 7 waves or more at up to 4 bits (row-streaming kernel,
-    // another 3-15 %) and M = 4 at 3 bits (4x4x4 kernel, 9 % on 4096 x 14336 and 8192 x 28672)
-    if (knob(kGemvRows) <= 0 && m4 <= 1 && q.geo->wpl == 1 && long_rows_want_four(M, K)) {
-        if (single(q) && M == 3 && b <= 4 && q.geo->S >= 7 && stream_ok) return AP_ROUTE_STREAM;
+    // long_rows_want_four says -- except M = 3 on rows of 8 waves or more at up to 4 bits (row-streaming kernel,
+    // another 3-15 %; rows of 7 waves are 0-7 % faster with four rows) and M = 4 at 3 bits (4x4x4 kernel, 9 % on
+    // 4096 x 14336 and 8192 x 28672)
+    if (knob(kGemvRows) <= 0 && m4 <= 1 && q.geo->wpl == 1 && long_rows_want_four(M, K, b)) {
+        if (single(q) && M == 3 && b <= 4 && q.geo->S >= 8 && stream_ok) return AP_ROUTE_STREAM;
         if (!(M == 4 && b == 3 && m4 == 1)) return AP_ROUTE_DOT;
     }
     if (single(q)) {
-        const bool wide = q.lo >= 8192 && K <= 4096;  // gate/up of the 7B / 8B models
-        // row-streaming kernel (fewest waves and instructions): 3 bits at one row on wide linears (3-5 %), 3-4 bits at
-        // two rows on rows of >= 8192 elements that long_rows_want_four left alone (10-14 %)
-        if (stream_ok && ((M == 1 && wide && b == 3) || (M == 2 && K >= 8192 && b <= 4))) return AP_ROUTE_STREAM;
-        // fine-grained row-pair kernel (half the waves): 6-7 bits at one row on wide linears (3-6 %; at 8 bits one row per
-        // workgroup of gemv_kbit_kernel is faster still), 6-8 bits at four rows on rows of >= 8192 elements (6-15 %; at
-        // 6 bits on rows of up to 12288 elements the 4x4x4 kernel is 13 % faster and takes over)
-        if (fine_ok && ((M == 1 && wide && (b == 6 || b == 7)) || (M == 4 && K >= 8192 && b >= (K <= 12288 ? 7 : 6))))
-            return AP_ROUTE_FINE;
+        // row-streaming kernel (fewest waves and instructions): 3-4 bits at two rows on rows of >= 8192 elements that
+        // long_rows_want_four left alone (10-14 %).  It also served 3 bits at one row on wide linears (3-5 % then); since
+        // the dot-product kernel's prologue was trimmed that kernel is 5-6 % faster there (11008 x 4096: 7.2 -> 6.8 us,
+        // 14336 x 4096: 8.3 -> 7.8).
+        if (stream_ok && M == 2 && K >= 8192 && b <= 4) return AP_ROUTE_STREAM;
+        // fine-grained row-pair kernel (half the waves): 6-8 bits at four rows on rows of >= 8192 elements (6-15 %; at
+        // 6 bits on rows of up to 12288 elements the 4x4x4 kernel is 13 % faster and takes over).  At one row it served
+        // 6-7 bits on wide linears (11008 / 14336 x 4096; 3-6 % then): the dot-product kernel with two rows per workgroup is
+        // now 3-6 % faster there (11008 x 4096 at 6 bits: 10.3 -> 9.7 us).
+        if (fine_ok && M == 4 && K >= 8192 && b >= (K <= 12288 ? 7 : 6)) return AP_ROUTE_FINE;
     }
     // The 4x4x4 matrix-core kernel (cost per weight flat in M, one linear per launch): 3 and 4 rows on single linears with
     // enough rows to fill the chip, at up to 5 bits, and for 4 rows at every bit-width while a row fits one word

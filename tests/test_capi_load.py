@@ -173,12 +173,14 @@ def test_route_report_follows_the_rule_and_the_knobs():
     """ap_matmul_kbit_route names the kernel a single linear gets; forcing knobs change it at once."""
     from any_precision_amd import _capi
     assert _capi.matmul_route(1, 4096, 4096, 4) == "dot"
-    assert _capi.matmul_route(1, 11008, 4096, 3) == "stream"
-    assert _capi.matmul_route(1, 11008, 4096, 7) == "fine"
+    assert _capi.matmul_route(1, 11008, 4096, 3) == "dot"
+    assert _capi.matmul_route(1, 11008, 4096, 7) == "dot" and _capi.matmul_route(4, 4096, 11008, 7) == "fine"
     assert _capi.matmul_route(1, 11008, 4096, 8) == "dot"
     assert _capi.matmul_geometry(1, 11008, 4096, 8)["rows"] == 1        # one row per workgroup at 8 bits
     assert _capi.matmul_route(1, 4096, 11008, 3) == "dot"
-    assert _capi.matmul_route(2, 4096, 14336, 4) == "stream"
+    assert _capi.matmul_route(2, 4096, 14336, 4) == "dot" and _capi.matmul_geometry(2, 4096, 14336, 4)["rows"] == 4
+    assert _capi.matmul_route(2, 8192, 28672, 4) == "stream"           # rows of 14 waves keep the streaming kernel
+    assert _capi.matmul_geometry(2, 4096, 4096, 3)["rows"] == 2 and _capi.matmul_geometry(2, 4096, 4096, 5)["rows"] == 1
     assert _capi.matmul_route(8, 4096, 4096, 4) == "mfma16"
     assert _capi.matmul_route(8, 14336, 4096, 4) == "mfma4"
     assert _capi.matmul_route(8, 14336, 4096, 3) == "mfma16"            # pair-table lookups: faster at 3 bits
