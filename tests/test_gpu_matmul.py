@@ -398,8 +398,11 @@ def test_four_rows_per_workgroup_agree_with_the_oracle(ext, oracle):
     assert _capi.matmul_geometry(1, 4096, 11008, 3)["rows"] == 2
     assert _capi.matmul_geometry(1, 4096, 4096, 3)["rows"] == 1
     assert _capi.matmul_geometry(2, 14336, 4096, 3)["rows"] == 2      # short rows: four only at one activation row
-    # 2..4 activation rows on long rows: four rows per workgroup, except rows of 5..6 waves at M = 3, 4 and of 7+ at M = 2
-    for M, N, K, rows, route in ((2, 4096, 11008, 4, "dot"), (2, 4096, 14336, 2, "stream"), (3, 4096, 14336, 4, "stream"),
+    # 2..4 activation rows on long rows: four rows per workgroup, except rows of 5..6 waves at M = 3, 4 and of 9+ at M = 2
+    # (7+ from 5 bits on); the row-streaming kernel keeps M = 3 at up to 4 bits on rows of 8 waves or more
+    assert _capi.matmul_geometry(2, 4096, 14336, 5)["rows"] == 2
+    for M, N, K, rows, route in ((2, 4096, 11008, 4, "dot"), (2, 4096, 14336, 4, "dot"), (3, 4096, 14336, 4, "dot"),
+                                 (3, 4096, 16384, 4, "stream"),
                                  (3, 8192, 8192, 4, "dot"), (3, 4096, 11008, 2, "mfma4"), (4, 5120, 13824, 4, "dot"),
                                  (4, 28672, 8192, 4, "dot")):
         assert _capi.matmul_geometry(M, N, K, 4)["rows"] == rows and _capi.matmul_route(M, N, K, 4) == route, (M, N, K)
