@@ -44,6 +44,7 @@ enum {
     kGemmTiled,         // tiled fused GEMM (ap_gemm_kbit): 0 never, 1 where it pays, 2 wherever it fits
     kGemmTile,          // > 0: blocks of 16 activation rows in its tile: 1, 2, 4 or 8
     kGemmTileSplit,     // > 0: groups of four waves per workgroup of the 64-row tile, each on its share of K: 1 or 2
+    kGemmLookahead,     // K-split fused GEMM, lookups one word ahead of the matrix instructions: 0 never, 1 where it pays, 2 wherever the variant exists
     kKnobCount
 };
 Knob g_knobs[kKnobCount] = {
@@ -52,7 +53,7 @@ Knob g_knobs[kKnobCount] = {
     {"gemm_rb2", 1},              {"gemv_stream", 1},    {"gemv_stream_waves", 24},
     {"gemv_fine", 1},
     {"gemm_walk", 1},             {"gemm_walk_wgs", 1},  {"gemm_tiled", 1},   {"gemm_tile", 0},
-    {"gemm_tile_split", 0},
+    {"gemm_tile_split", 0},       {"gemm_lookahead", 1},
 };
 inline int knob(int k) { return __atomic_load_n(&g_knobs[k].value, __ATOMIC_RELAXED); }
 
@@ -550,6 +551,13 @@ int run_gemm(const uint16_t *x, const uint32_t *qweight, const uint16_t *lut, ui
     if (ks > steps) ks = steps;
     if (ks < 1) ks = 1;
     geo.ks = ks;
+    // Lookups one word ahead of the matrix instructions where a CU holds one workgroup and nothing else covers a
+    // wave's waits for its lookups (4096-row linears: 2-7 %); with several workgroups per CU the same variant is 5-20 %
+    // slower, and at 8 bits with one step per wave and one block of activation rows 3-4 % (4096 x 4096).
+    const int la_mode = knob(kGemmLookahead);
+    const bool la_fits = geo.rb == 1 && geo.mb <= 2 && (W & 3) == 0;
+    const bool la_pays = geo.grid <= cu_count() && !(w_bits == 8 && geo.mb == 1 && steps <= ks);
+    geo.lookahead = la_fits && (la_mode >= 2 || (la_mode == 1 && la_pays)) ? 1 : 0;
     switch (w_bits) {
         case 3: launch_gemm<3>(geo, x, qweight, lut, out, M, N, K, st); break;
         case 4: launch_gemm<4>(geo, x, qweight, lut, out, M, N, K, st); break;

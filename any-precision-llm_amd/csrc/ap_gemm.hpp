@@ -61,7 +61,8 @@ __device__ __forceinline__ void transpose_rows4(uint32_t (&r)[4]) {
 // lockstep: every activation operand it loads then feeds RB matrix instructions instead of one,
 // which divides the L2 traffic of the activations by RB -- at the price of 1/RB as many
 // workgroups, so only linears with many rows use RB = 2.  Grid: ceil(N / (16 RB)) workgroups of (64, KS).
-template <int BITS, int MB, bool VEC4, int MP, int RB>
+// LOOKAHEAD: see the step below.
+template <int BITS, int MB, bool VEC4, int MP, int RB, bool LOOKAHEAD = false>
 __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
     half_t *__restrict__ out, int M, int N, int K, int KS, uint32_t ks_magic) {
@@ -132,12 +133,42 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
         }
     };
 
-    // Load order: planes of the first step, then the tables -- both are in flight together
-    // and the tables are staged while nothing else could run anyway.  The tables of the
+    // byte offset of this lane's activation row in each row block (rows past M repeat row M-1)
+    uint32_t xoff[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) xoff[mb] = (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)K * 2u;
+    const int full_chunks = W >> 5;                // chunks of 32 words; a shorter one may follow
+    const uint32_t tail_stride = (uint32_t)(W & 31) * 16u;  // bytes of x between byte groups in the tail chunk
+    // x byte offset (within a row) of byte group j of the wi-th word of this lane in `step`; a word past the row
+    // end takes the last word's
+    auto a_offset = [&](int step, int wi, int j) {
+        const int w = min(4 * (WPS * step + wi) + grp, W - 1);
+        const int chunk = w >> 5;
+        return ((uint32_t)chunk << 11) + ((uint32_t)(w & 31) << 4) + (uint32_t)j * (chunk == full_chunks ? tail_stride : 512u);
+    };
+    // The unit of the inner schedule is the octet (one byte group of one word: one B operand,
+    // MB MFMAs).  Its A operand is 16 bytes of x per lane, lane (m, g) taking row m and the
+    // g-th octet of a 64-byte run.  Every workgroup reads its K-slices of ALL of x, so the
+    // activations are re-read N/16 times from L2 -- (N/16) * M * K * 2 bytes, more than the
+    // planes from M = 2 * w_bits rows on.
+    // MP == 0: the operands are loaded straight from global memory, AHEAD octets early.  (Requesting all sixteen
+    // of a step at once, with the planes or right after the tables, measured slower: so many loads whose lanes
+    // sit in sixteen different rows delay the plane data that every wave waits for first.)
+    // MP > 0: the wave loads the x block of a word group (MP rows x 4 runs of 64 bytes) with
+    // adjacent lanes on adjacent addresses, parks it in its own LDS region and reads the
+    // operands from there (slots skewed by the octet index so that writes and reads are free
+    // of bank conflicts; LDS operations of one wave complete in order, so no barrier).
+    constexpr int OCT = 4 * WPS;
+    constexpr int AHEAD = MB == 1 ? 4 : (MB == 2 ? 2 : 1);
+    constexpr int NL = MP / 4;  // staging loads per lane and word group
+
+    // Load order: planes of the first step, then the tables -- both in flight
+    // together, and the tables are staged while nothing else could run anyway.  The tables of the
     // workgroup's rows are contiguous in lut (rows past N re-read the last 16 bytes of the
     // array; their columns are never stored).
-    uint32_t qn[RB][BITS][WPS];
-    if (s_begin < s_end) fetch(s_begin, qn);
+    // (every wave has at least one step: the host launches at most as many waves as there are steps)
+    uint32_t qa[RB][BITS][WPS], qb[RB][BITS][WPS];
+    fetch(s_begin, qa);
     if constexpr (PAIR) {
         // wave ks builds the pair tables of rows ks, ks + KS, ...: the loads of the first ROWS / 8 of them (all,
         // when the workgroup has its eight waves) are issued together
@@ -167,13 +198,6 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
     typedef __attribute__((address_space(3))) uint32_t lds_u32_t;
     const uint32_t tab_base0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t *)&tables[0][0]) + (uint32_t)col * TB;
 
-    // byte offset of this lane's activation row in each row block (rows past M repeat row M-1)
-    uint32_t xoff[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++) xoff[mb] = (uint32_t)min(mb * 16 + col, M - 1) * (uint32_t)K * 2u;
-    const int full_chunks = W >> 5;                // chunks of 32 words; a shorter one may follow
-    const uint32_t tail_stride = (uint32_t)(W & 31) * 16u;  // bytes of x between byte groups in the tail chunk
-
     float4_t acc[RB][MB];
 #pragma unroll
     for (int rb = 0; rb < RB; rb++)
@@ -182,41 +206,23 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 
     // One step: transpose the planes of each word to indices, gather, multiply.  CHECK: the
     // step may reach past the end of the row (only the last step of a row can).
-    //
-    // The unit of the inner schedule is the octet (one byte group of one word: one B operand,
-    // MB MFMAs).  Its A operand is 16 bytes of x per lane, lane (m, g) taking row m and the
-    // g-th octet of a 64-byte run.  Every workgroup reads its K-slices of ALL of x, so the
-    // activations are re-read N/16 times from L2 -- (N/16) * M * K * 2 bytes, more than the
-    // planes from M = 2 * w_bits rows on -- and that traffic, not HBM, bounds the kernel.
-    // MP == 0: the operands are loaded straight from global memory, AHEAD octets early.
-    // MP > 0: the wave loads the x block of a word group (MP rows x 4 runs of 64 bytes) with
-    // adjacent lanes on adjacent addresses, parks it in its own LDS region and reads the
-    // operands from there (slots skewed by the octet index so that writes and reads are free
-    // of bank conflicts; LDS operations of one wave complete in order, so no barrier).
-    constexpr int OCT = 4 * WPS;
-    constexpr int AHEAD = MB == 1 ? 4 : (MB == 2 ? 2 : 1);
-    constexpr int NL = MP / 4;  // staging loads per lane and word group
+    // LOOKAHEAD: the lookups run one word ahead of the matrix instructions -- the 16 (pair tables) or 32 gathers
+    // of word wi + 1 are issued before the four octets of word wi are multiplied (a second set of B operands), so
+    // the wave waits for LDS once per word and not once per octet.  Measured 2-9 % faster where a CU holds one
+    // workgroup (linears of up to 16 rows per CU), and 5-20 % slower where it holds several, whose waves cover
+    // each other's waits and lose occupancy to the extra registers: the host chooses.
     auto process = [&](auto check_c, int step, uint32_t(&q)[RB][BITS][WPS]) {
         constexpr bool CHECK = decltype(check_c)::value;
-        // x byte offset of byte group 0 of each word, and the distance between byte groups
-        uint32_t kb[WPS], jstride[WPS];
         bool live[WPS];
 #pragma unroll
-        for (int wi = 0; wi < WPS; wi++) {
-            const int w = 4 * (WPS * step + wi) + grp;
-            live[wi] = !CHECK || w < W;  // words past the row end contribute zeros
-            const int wc = live[wi] ? w : W - 1;
-            const int chunk = wc >> 5;
-            kb[wi] = ((uint32_t)chunk << 11) + ((uint32_t)(wc & 31) << 4);
-            jstride[wi] = chunk == full_chunks ? tail_stride : 512u;
-        }
+        for (int wi = 0; wi < WPS; wi++) live[wi] = !CHECK || 4 * (WPS * step + wi) + grp < W;  // words past the row end contribute zeros
 
         // ---- direct path (MP == 0): fragments from global memory, AHEAD octets early
         half8_t a[MP == 0 ? OCT : 1][MB];
         auto load_a = [&](auto t_c) {
             constexpr int t = decltype(t_c)::value;
             if constexpr (MP == 0 && t < OCT) {
-                const uint32_t koff = kb[t / 4] + (uint32_t)(t % 4) * jstride[t / 4];
+                const uint32_t koff = a_offset(step, t / 4, t % 4);
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
                     a[t][mb] = load_at<half8_t>(xg, xoff[mb] + koff);
@@ -248,6 +254,59 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
             }
         };
 
+        // B operands in flight: bws[slot][j][rb] = the eight weights of byte group j (LOOKAHEAD: slot = word & 1)
+        u32x4 bws[LOOKAHEAD ? 2 : 1][LOOKAHEAD ? 4 : 1][RB];
+        // index bytes hold the byte offset into the table (index * 2) where that fits a byte
+        constexpr int PRE = BITS <= 7 ? 1 : 0;
+        uint32_t idx[LOOKAHEAD ? 2 : 1][RB][PAIR ? 4 : 8];
+        auto indices = [&](auto wi_c) {
+            constexpr int wi = decltype(wi_c)::value, slot = LOOKAHEAD ? wi & 1 : 0;
+#pragma unroll
+            for (int rb = 0; rb < RB; rb++) {
+                uint32_t qq[BITS];
+#pragma unroll
+                for (int p = 0; p < BITS; p++) qq[p] = q[rb][p][wi];
+                if constexpr (PAIR) planes_to_adjacent_pairs<BITS>(qq, idx[slot][rb]);
+                else planes_to_indices<BITS, PRE>(qq, idx[slot][rb]);
+            }
+        };
+        auto gather = [&](auto wi_c, auto j_c) {
+            constexpr int wi = decltype(wi_c)::value, j = decltype(j_c)::value, c = 3 - j, slot = LOOKAHEAD ? wi & 1 : 0;
+            static_for<RB>([&](auto rb_c) {
+                constexpr int rb = decltype(rb_c)::value;
+                const uint32_t tab_base = tab_base0 + rb * (kGemmRows * TB);
+                static_for<4>([&](auto e_c) {
+                    constexpr int i = decltype(e_c)::value;
+                    uint32_t packed;
+                    if constexpr (PAIR) {
+                        // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
+                        uint32_t a0;
+                        if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[slot][rb][i]);
+                        else a0 = tab_base + byte_offset<c, 2>(idx[slot][rb][i]);
+                        packed = *reinterpret_cast<const lds_u32_t *>(a0);
+                    } else {
+                        uint32_t a0, a1;
+                        if constexpr (PRE) {
+                            a0 = byte_add<c>(tab_base, idx[slot][rb][2 * i]);
+                            a1 = byte_add<c>(tab_base, idx[slot][rb][2 * i + 1]);
+                        } else {
+                            a0 = tab_base + byte_offset<c, 1>(idx[slot][rb][2 * i]);
+                            a1 = tab_base + byte_offset<c, 1>(idx[slot][rb][2 * i + 1]);
+                        }
+                        half2_t h;
+                        h.x = *reinterpret_cast<const lds_half_t *>(a0);
+                        h.y = *reinterpret_cast<const lds_half_t *>(a1);
+                        packed = __builtin_bit_cast(uint32_t, h);
+                    }
+                    bws[slot][LOOKAHEAD ? j : 0][rb][i] = live[wi] ? packed : 0u;
+                });
+            });
+        };
+        auto lookups = [&](auto wi_c) {  // a whole word
+            indices(wi_c);
+            static_for<4>([&](auto j_c) { gather(wi_c, j_c); });
+        };
+
         if constexpr (MP > 0) stage_load(0);
         static_for<AHEAD>([&](auto t_c) { load_a(t_c); });
         if constexpr (VEC4) {
@@ -256,100 +315,70 @@ __global__ __launch_bounds__(kGemmMaxSplit *kWave) void gemm_kbit_kernel(
 #pragma unroll
                 for (int p = 0; p < BITS; p++) transpose_rows4(q[rb][p]);
         }
-        // index bytes hold the byte offset into the table (index * 2) where that fits a byte
-        constexpr int PRE = BITS <= 7 ? 1 : 0;
-        uint32_t idx[RB][PAIR ? 4 : 8];
-        static_for<OCT>([&](auto t_c) {
-            constexpr int t = decltype(t_c)::value, wi = t / 4, j = t % 4, c = 3 - j;
-            load_a(std::integral_constant<int, t + AHEAD>{});
-            if constexpr (j == 0) {
-                if constexpr (MP > 0) {
-                    stage_store();
-                    if constexpr (wi + 1 < WPS) stage_load(wi + 1);
-                }
-#pragma unroll
-                for (int rb = 0; rb < RB; rb++) {
-                    uint32_t qq[BITS];
-#pragma unroll
-                    for (int p = 0; p < BITS; p++) qq[p] = q[rb][p][wi];
-                    if constexpr (PAIR) planes_to_adjacent_pairs<BITS>(qq, idx[rb]);
-                    else planes_to_indices<BITS, PRE>(qq, idx[rb]);
-                }
+        if constexpr (LOOKAHEAD) lookups(std::integral_constant<int, 0>{});
+        static_for<WPS>([&](auto wi_c) {
+            constexpr int wi = decltype(wi_c)::value;
+            if constexpr (MP > 0) {
+                stage_store();
+                if constexpr (wi + 1 < WPS) stage_load(wi + 1);
             }
-            // B operands: the eight weights of byte group j of each row block
-            half8_t bfrag[RB];
-            static_for<RB>([&](auto rb_c) {
-                constexpr int rb = decltype(rb_c)::value;
-                const uint32_t tab_base = tab_base0 + rb * (kGemmRows * TB);
-                u32x4 bw;
-                static_for<4>([&](auto e_c) {
-                    constexpr int i = decltype(e_c)::value;
-                    uint32_t packed;
-                    if constexpr (PAIR) {
-                        // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
-                        uint32_t a0;
-                        if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[rb][i]);
-                        else a0 = tab_base + byte_offset<c, 2>(idx[rb][i]);
-                        packed = *reinterpret_cast<const lds_u32_t *>(a0);
+            if constexpr (!LOOKAHEAD) indices(wi_c);
+            else if constexpr (wi + 1 < WPS) lookups(std::integral_constant<int, wi + 1>{});
+            if constexpr (LOOKAHEAD) __builtin_amdgcn_sched_barrier(0);  // keeps the gathers of word wi + 1 ahead of the multiplications of word wi
+            static_for<4>([&](auto j_c) {
+                constexpr int j = decltype(j_c)::value, t = 4 * wi + j;
+                load_a(std::integral_constant<int, t + AHEAD>{});
+                if constexpr (!LOOKAHEAD) gather(wi_c, j_c);
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    half8_t afrag;
+                    if constexpr (MP > 0) {
+                        const int o = 4 * j + grp;
+                        const int m = (mb * 16 + col) & (MP - 1);  // MP < 16: rows repeat, their results are not stored
+                        afrag = __builtin_bit_cast(half8_t, xs[ks][o * MP + ((m + o) & (MP - 1))]);
                     } else {
-                        uint32_t a0, a1;
-                        if constexpr (PRE) {
-                            a0 = byte_add<c>(tab_base, idx[rb][2 * i]);
-                            a1 = byte_add<c>(tab_base, idx[rb][2 * i + 1]);
-                        } else {
-                            a0 = tab_base + byte_offset<c, 1>(idx[rb][2 * i]);
-                            a1 = tab_base + byte_offset<c, 1>(idx[rb][2 * i + 1]);
-                        }
-                        half2_t h;
-                        h.x = *reinterpret_cast<const lds_half_t *>(a0);
-                        h.y = *reinterpret_cast<const lds_half_t *>(a1);
-                        packed = __builtin_bit_cast(uint32_t, h);
+                        afrag = a[t][mb];
                     }
-                    bw[i] = live[wi] ? packed : 0u;
-                });
-                bfrag[rb] = __builtin_bit_cast(half8_t, bw);
+                    // words past the row end: zero activations as well as zero weights (0 * inf would be NaN)
+                    if constexpr (CHECK) {
+                        if (!live[wi]) afrag = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+                    }
+#pragma unroll
+                    for (int rb = 0; rb < RB; rb++)
+                        acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, __builtin_bit_cast(half8_t, bws[LOOKAHEAD ? wi & 1 : 0][LOOKAHEAD ? j : 0][rb]),
+                                                                             acc[rb][mb], 0, 0, 0);
+                }
             });
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
-                half8_t afrag;
-                if constexpr (MP > 0) {
-                    const int o = 4 * j + grp;
-                    const int m = (mb * 16 + col) & (MP - 1);  // MP < 16: rows repeat, their results are not stored
-                    afrag = __builtin_bit_cast(half8_t, xs[ks][o * MP + ((m + o) & (MP - 1))]);
-                } else {
-                    afrag = a[t][mb];
-                }
-                // words past the row end: zero activations as well as zero weights (0 * inf would be NaN)
-                if constexpr (CHECK) {
-                    if (!live[wi]) afrag = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-                }
-#pragma unroll
-                for (int rb = 0; rb < RB; rb++)
-                    acc[rb][mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(afrag, bfrag[rb], acc[rb][mb], 0, 0, 0);
-            }
         });
     };
 
-    // With few planes the next step's words are fetched while this step computes; with
-    // many, the second register set is not worth its registers (no measurable gain).
-    constexpr bool PREFETCH = RB * BITS * WPS <= 20;
-    for (int step = s_begin; step < s_end; step++) {
-        uint32_t q[RB][BITS][WPS];
-        if (PREFETCH || step == s_begin) {
-#pragma unroll
-            for (int rb = 0; rb < RB; rb++)
-#pragma unroll
-                for (int p = 0; p < BITS; p++)
-#pragma unroll
-                    for (int i = 0; i < WPS; i++) q[rb][p][i] = qn[rb][p][i];
-        } else {
-            fetch(step, q);
-        }
-        if (PREFETCH && step + 1 < s_end) fetch(step + 1, qn);
+    auto run = [&](int step, uint32_t(&q)[RB][BITS][WPS]) {
         if (4 * WPS * (step + 1) <= W)
             process(std::false_type{}, step, q);
         else
             process(std::true_type{}, step, q);
+    };
+    // With few planes the next step's words are fetched while this step computes, two register sets taking turns
+    // (the loop body is written out twice: handing the prefetched registers over with copies makes the wave wait
+    // for those loads where the copies stand); with many, the second set is not worth its registers (no
+    // measurable gain) and a step's words are fetched when the step before it is done.
+    constexpr bool PREFETCH = RB * BITS * WPS <= 20;
+    int step = s_begin;
+    if constexpr (PREFETCH) {
+        for (;;) {
+            if (step + 1 < s_end) fetch(step + 1, qb);
+            run(step, qa);
+            if (++step >= s_end) break;
+            if (step + 1 < s_end) fetch(step + 1, qa);
+            run(step, qb);
+            if (++step >= s_end) break;
+        }
+    } else {
+        for (;;) {
+            run(step, qa);
+            if (++step >= s_end) break;
+            fetch(step, qa);
+        }
     }
 
     // Combine the K-split partial tiles in wave order (also with one wave: it keeps the

@@ -28,6 +28,11 @@ void launch_gemm(const GemmGeometry &geo, const uint16_t *x, const uint32_t *qwe
         else gemm_kbit_kernel<BITS, 2, true, 32, 2><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);
         return;
     }
+    if (geo.lookahead && vec4 && geo.mb <= 2) {
+        if (geo.mb == 1) gemm_kbit_kernel<BITS, 1, true, 0, 1, true><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);
+        else gemm_kbit_kernel<BITS, 2, true, 32, 1, true><<<grid, block, 0, stream>>>(xh, qweight, lh, oh, M, N, K, geo.ks, ks_magic);
+        return;
+    }
     switch (geo.mb) {
         AP_GEMM_CASE(1)
         case 2: AP_GEMM_LAUNCH(2, 32); break;

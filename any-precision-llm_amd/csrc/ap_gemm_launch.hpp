@@ -14,6 +14,7 @@ struct GemmGeometry {
     int ks;    // K-split waves per workgroup
     int rb;    // blocks of 16 weight rows per workgroup: 1, or 2 (only with K % 128 == 0 and mb <= 2)
     int grid;  // workgroups = ceil(N / (16 rb))
+    int lookahead;  // 1: gathers one word ahead of the matrix instructions (one or two activation row blocks, rb = 1, K % 128 == 0)
 };
 
 // Launches gemm_kbit_kernel<BITS, geo.mb, ..., geo.rb> on `stream`.

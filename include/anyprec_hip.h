@@ -165,7 +165,7 @@ int ap_matmul_kbit_group_route(int count, const int *N, int M, int K, int w_bits
  * beyond the 1e-2 bar of the entry points; the defaults are what measured fastest.  Names:
  * gemv_target_waves, gemv_rows, gemv_wpl, dequant_blocks_per_cu, matmul_mfma_from, gemm_split,
  * matmul_mfma4, gemv4_groups, gemm_rb2, gemv_stream, gemv_stream_waves, gemv_fine,
- * gemm_walk, gemm_walk_wgs, gemm_tiled, gemm_tile, gemm_tile_split.  Returns AP_OK, AP_ENULL or AP_EKNOB.
+ * gemm_walk, gemm_walk_wgs, gemm_tiled, gemm_tile, gemm_tile_split, gemm_lookahead.  Returns AP_OK, AP_ENULL or AP_EKNOB.
  * For tests and measurements only: the knobs are plain process-wide integers, NOT thread-safe against
  * concurrent launches (a launch that races with a change sees either value); a serving process leaves
  * them alone. */

@@ -158,7 +158,8 @@ def test_tuning_knobs_need_no_gpu():
     with pytest.raises(ValueError):
         _capi.get_tuning("no_such_knob")
     for name in ("gemv_target_waves", "gemv_rows", "gemv_wpl", "dequant_blocks_per_cu", "matmul_mfma_from", "gemm_split",
-                 "matmul_mfma4", "gemv4_groups", "gemm_rb2", "gemv_stream", "gemv_stream_waves", "gemv_fine"):
+                 "matmul_mfma4", "gemv4_groups", "gemm_rb2", "gemv_stream", "gemv_stream_waves", "gemv_fine",
+                 "gemm_walk", "gemm_walk_wgs", "gemm_tiled", "gemm_tile", "gemm_tile_split", "gemm_lookahead"):
         before = _capi.get_tuning(name)
         with _capi.tuning(**{name: before + 3}):
             assert _capi.get_tuning(name) == before + 3

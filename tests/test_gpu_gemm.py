@@ -154,6 +154,28 @@ def test_two_weight_row_blocks_per_workgroup_give_the_same_bits(ext, oracle):
                 assert torch.equal(plain.view(torch.int16), forced.view(torch.int16)), (N, K, b, M)
 
 
+def test_lookups_one_word_ahead_give_the_same_bits(ext, oracle):
+    """Linears of up to 16 rows per CU run the K-split kernel with its table lookups one word ahead of the matrix
+    instructions; the knob gemm_lookahead switches the variant off (0) or forces it wherever it exists (2).  The
+    order of the additions does not change, so both must give the same bits; rows of 344 and 448 words end in a
+    partial step."""
+    from any_precision_amd import _capi
+    for N, K in ((33, 1024), (47, 2176), (176, 11008), (144, 14336), (32, 128)):
+        L = make(N, K, seed=N + K)
+        q, luts = layer_to_gpu(L)
+        for b in range(3, 9):
+            for M in (5, 9, 16, 20, 32):
+                print(f"lookahead N={N} K={K} b={b} M={M}", flush=True)
+                x, xg = _x(M, K, seed=M)
+                with _capi.tuning(gemm_lookahead=2, gemm_rb2=0, gemm_tiled=0, gemm_walk=0):
+                    ahead = ext.gemm_kbit(xg, q, luts[b], b)
+                _, want = oracle.matmul_kbit(x, L.qweight, L.luts[b], b, return_f64=True)
+                assert_close_gemv(ahead, want, f"N={N} K={K} b={b} M={M}")
+                with _capi.tuning(gemm_lookahead=0, gemm_rb2=0, gemm_tiled=0, gemm_walk=0):
+                    plain = ext.gemm_kbit(xg, q, luts[b], b)
+                assert torch.equal(plain.view(torch.int16), ahead.view(torch.int16)), (N, K, b, M)
+
+
 def test_row_walking_kernel_agrees_with_the_oracle(ext, oracle):
     """Wide linears at up to 32 activation rows run a variant whose workgroups walk the blocks of weight rows
     with their activations held in registers; the knob gemm_walk = 2 forces it wherever it fits (rows of a
