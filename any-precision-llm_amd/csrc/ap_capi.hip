@@ -778,11 +778,12 @@ void many_rows_route(const RouteQuery &q, int *route) {
         return;
     }
     // 4x4x4 kernel with two groups of four activation rows (5..8 rows): on wide linears (16 rows per workgroup) with
-    // rows of 3072..4096 elements (5..8 waves per workgroup) from 4 bits on it is 5-20 % faster than the 16x16x32
-    // kernel; shorter and longer rows and narrower linears measured slower, and at 3 bits the 16x16x32 kernel with its
-    // pair-table lookups is 4-18 % faster (11008 / 14336 x 4096).
+    // rows of 3072..4096 elements (5..8 waves per workgroup) from 5 bits on it is 5-20 % faster than the 16x16x32
+    // kernel; shorter and longer rows and narrower linears measured slower, and at 3 and 4 bits the 16x16x32 kernel
+    // with its pair-table lookups is 4-18 % faster (11008 / 14336 x 4096; at 4 bits 6-12 % since its lookups run ahead
+    // and its plane loads no longer wait).
     for (int g = 0; g < q.count; g++) {
-        const bool pays = q.M >= 5 && q.K >= 3072 && q.N[g] >= 10240 && q.w_bits >= 4;
+        const bool pays = q.M >= 5 && q.K >= 3072 && q.N[g] >= 10240 && q.w_bits >= 5;
         route[g] = m4 >= 1 && mfma4_fits(q) && (m4 >= 2 || pays) ? AP_ROUTE_MFMA4 : AP_ROUTE_MFMA16;
     }
 }

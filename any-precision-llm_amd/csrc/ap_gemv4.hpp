@@ -33,6 +33,7 @@
 #include "ap_bitplane.hpp"
 #include "ap_device.hpp"
 #include "ap_gemv4_launch.hpp"
+#include "ap_lookup.hpp"
 
 namespace ap {
 
@@ -49,9 +50,11 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     constexpr int MAXS = THREADS / kWave;
     constexpr int MR = 4 * MG;  // activation rows computed (rows past M repeat row M-1 and are not stored)
     constexpr int ROWS = 4 * RQ;
-    // plain tables at every bit-width: pair tables (two weights per entry, as in the dot-product
-    // kernel) measured equal or slower here, the permuted activations cost what the packing saves
-    constexpr int TB = 2 << BITS;
+    // 3 and 4 bits: tables of the weights of two ADJACENT elements (ap_lookup.hpp) -- one 32-bit gather per half of a
+    // B operand, no packing of two 16-bit gathers, and the entry numbers come out of a shorter transpose
+    // (planes_to_adjacent_pairs).  The activations stay as they sit in memory.
+    constexpr bool PAIR = LookupTable<BITS>::kPair;
+    constexpr int TB = LookupTable<BITS>::kBytes;
     __shared__ __attribute__((aligned(16))) uint8_t tables[ROWS][TB];
     __shared__ float partial[MAXS][ROWS][MR];  // [wave][weight row][activation row]
 
@@ -69,10 +72,11 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     // activations.
     // table r is staged by wave r & (P - 1), P = largest power of two <= S
     const int pmask = (1 << (31 - __builtin_clz(S))) - 1;
-    LutRegs<BITS> t[ROWS];
+    const PairLane<BITS> pl = pair_lane<BITS>(lane);
+    TableWords<BITS> t[ROWS];
 #pragma unroll
     for (int r = 0; r < ROWS; r++)
-        if (s == (r & pmask)) t[r] = lut_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane);
+        if (s == (r & pmask)) t[r] = lookup_table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane, pl);
 
     uint32_t q[RQ][G][BITS];
     bool live[G];
@@ -124,13 +128,20 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
 
 #pragma unroll
     for (int r = 0; r < ROWS; r++)
-        if (s == (r & pmask)) lut_stage<BITS>(t[r], reinterpret_cast<half_t *>(tables[r]), lane);
+        if (s == (r & pmask)) {
+            lookup_table_arrive<BITS>(t[r]);
+            lookup_table_stage<BITS>(t[r], tables[r], lane);
+        }
     if (S > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
 
     // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
     typedef __attribute__((address_space(3))) uint8_t lds_byte_t;
     const uint32_t tab_base0 = (uint32_t)(uintptr_t)((lds_byte_t *)&tables[0][0]) + (uint32_t)qi * TB;
 
+    // CHECK: this wave's words may reach past the row end (the last wave of a row only); every other wave runs the copy
+    // without the per-lookup selects (a scalar branch).
+    auto compute = [&](auto check_c) {
+    constexpr bool CHECK = decltype(check_c)::value;
     static_for<RQ>([&](auto rq_c) {
     constexpr int rq = decltype(rq_c)::value;
     const uint32_t tab_base = tab_base0 + rq * 4 * TB;
@@ -145,26 +156,37 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
         for (int p = 0; p < BITS; p++) qq[p] = (uint32_t)__builtin_amdgcn_ds_bpermute(take, (int)q[rq][g][p]);
         // index bytes hold the byte offset into the table (index * 2) where that fits a byte
         constexpr int PRE = BITS <= 7 ? 1 : 0;
-        uint32_t idx[8];
-        planes_to_indices<BITS, PRE>(qq, idx);
+        uint32_t idx[PAIR ? 4 : 8];
+        if constexpr (PAIR) planes_to_adjacent_pairs<BITS>(qq, idx);
+        else planes_to_indices<BITS, PRE>(qq, idx);
         static_for<4>([&](auto j_c) {
             constexpr int j = decltype(j_c)::value, c = 3 - j;
             uint32_t bw[4];  // the eight weights of byte group j, two per register
             static_for<4>([&](auto e_c) {
                 constexpr int i = decltype(e_c)::value;
-                uint32_t a0, a1;
-                if constexpr (PRE) {
-                    a0 = byte_add<c>(tab_base, idx[2 * i]);
-                    a1 = byte_add<c>(tab_base, idx[2 * i + 1]);
+                uint32_t packed;
+                if constexpr (PAIR) {
+                    // byte c of idx[i]: the entry of elements (2i, 2i+1) of byte group j -- at 3 bits already its byte offset
+                    uint32_t a0;
+                    if constexpr (BITS == 3) a0 = byte_add<c>(tab_base, idx[i]);
+                    else a0 = tab_base + byte_offset<c, 2>(idx[i]);
+                    packed = *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>(a0);
                 } else {
-                    a0 = tab_base + byte_offset<c, 1>(idx[2 * i]);
-                    a1 = tab_base + byte_offset<c, 1>(idx[2 * i + 1]);
+                    uint32_t a0, a1;
+                    if constexpr (PRE) {
+                        a0 = byte_add<c>(tab_base, idx[2 * i]);
+                        a1 = byte_add<c>(tab_base, idx[2 * i + 1]);
+                    } else {
+                        a0 = tab_base + byte_offset<c, 1>(idx[2 * i]);
+                        a1 = tab_base + byte_offset<c, 1>(idx[2 * i + 1]);
+                    }
+                    const uint32_t lo = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a0);
+                    const uint32_t hi = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a1);
+                    packed = lo | (hi << 16);
                 }
-                const uint32_t lo = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a0);
-                const uint32_t hi = *reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(a1);
                 // words past the row end: zero weights as well as zero activations, so that a non-finite
                 // table entry or activation there cannot turn 0 * inf into NaN
-                bw[i] = live[g] ? (lo | (hi << 16)) : 0u;
+                bw[i] = !CHECK || live[g] ? packed : 0u;
             });
 #pragma unroll
             for (int h = 0; h < 2; h++) {
@@ -206,6 +228,11 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
         if ((lane & 15) >= 12) partial[s][4 * rq + qi][mg * 4 + which] = u;
     }
     });
+    };
+    // (only the variant of one word group and four activation rows has the registers for two copies: the others
+    // would cross a step of the occupancy table)
+    if (G > 1 || MG > 1 || (s * G + G) * 16 > W) compute(std::true_type{});
+    else compute(std::false_type{});
     __syncthreads();
     for (int o = s * kWave + lane; o < ROWS * MR; o += S * kWave) {
         const int m = o % MR, r = o / MR;

@@ -183,7 +183,7 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_route(2, 8192, 28672, 4) == "stream"           # rows of 14 waves keep the streaming kernel
     assert _capi.matmul_geometry(2, 4096, 4096, 3)["rows"] == 2 and _capi.matmul_geometry(2, 4096, 4096, 5)["rows"] == 1
     assert _capi.matmul_route(8, 4096, 4096, 4) == "mfma16"
-    assert _capi.matmul_route(8, 14336, 4096, 4) == "mfma4"
+    assert _capi.matmul_route(8, 14336, 4096, 5) == "mfma4" and _capi.matmul_route(8, 14336, 4096, 4) == "mfma16"
     assert _capi.matmul_route(8, 14336, 4096, 3) == "mfma16"            # pair-table lookups: faster at 3 bits
     assert _capi.matmul_route(8, 1024, 4096, 3) == "dot"                # too few rows for 16 per workgroup
     assert _capi.matmul_route(5, 5120, 5120, 8) == "dot" and _capi.matmul_route(8, 8192, 8192, 8) == "mfma16"
@@ -193,7 +193,7 @@ def test_route_report_follows_the_rule_and_the_knobs():
     assert _capi.matmul_group_route(1, [4096, 4096, 4096], 4096, 8) == (["dot"] * 3, 1)
     assert _capi.matmul_group_route(3, [4096, 1024, 1024], 4096, 5) == (["dot"] * 3, 4)
     assert _capi.matmul_group_route(8, [4096, 1024, 1024], 4096, 3)[0] == ["dot"] * 3       # a narrow member
-    assert _capi.matmul_group_route(8, [11008, 11008], 4096, 4)[0] == ["mfma4", "mfma4"]     # a launch per member
+    assert _capi.matmul_group_route(8, [11008, 11008], 4096, 5)[0] == ["mfma4", "mfma4"]     # a launch per member
     assert _capi.matmul_group_route(8, [4096, 4096, 4096], 4096, 3)[0] == ["mfma16"] * 3
     assert _capi.matmul_group_route(8, [8192, 1024, 1024], 8192, 3)[0] == ["mfma16", "dot", "dot"]   # each as a linear of its own
     with pytest.raises(ValueError):
