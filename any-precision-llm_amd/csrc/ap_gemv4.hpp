@@ -41,11 +41,12 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // MG = groups of four activation rows (M <= 4 MG), G = word groups per wave, RQ = row quads
-// per workgroup.  Grid: ceil(N / (4 RQ)) workgroups of (64, S) threads, S * 64 <= THREADS.
+// per workgroup.  Grid: ceil(N / (4 RQ)) workgroups of (64, S) threads, S * 64 <= THREADS (S is also an argument: it
+// arrives with the others instead of through a load of its own from the dispatch packet).
 template <int BITS, int MG, int G, int RQ, int THREADS>
 __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     const half_t *__restrict__ x, const uint32_t *__restrict__ qweight, const half_t *__restrict__ lut,
-    half_t *__restrict__ out, int M, int N, int K) {
+    half_t *__restrict__ out, int M, int N, int K, int S) {
     constexpr int NC = 1 << BITS;
     constexpr int MAXS = THREADS / kWave;
     constexpr int MR = 4 * MG;  // activation rows computed (rows past M repeat row M-1 and are not stored)
@@ -58,8 +59,11 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     __shared__ __attribute__((aligned(16))) uint8_t tables[ROWS][TB];
     __shared__ float partial[MAXS][ROWS][MR];  // [wave][weight row][activation row]
 
+    // every argument in scalar registers by one clause of scalar loads and one wait (the compiler alone loads an
+    // argument where it is first used: a dependent round trip to the scalar cache each)
+    asm volatile("" : "+s"(x), "+s"(qweight), "+s"(lut), "+s"(out), "+s"(M), "+s"(N), "+s"(K), "+s"(S));
     const int lane = threadIdx.x;
-    const int s = __builtin_amdgcn_readfirstlane(threadIdx.y), S = blockDim.y;
+    const int s = __builtin_amdgcn_readfirstlane(threadIdx.y);
     const int qi = lane & 3, wb = lane >> 2;
     const int W = K >> 5;
     const size_t plane_bytes = (size_t)N * W * sizeof(uint32_t);  // below 2^32 (the host checks)
@@ -70,13 +74,17 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
 
     // Load order as in the dot-product kernel: tables, planes (non-temporal: streamed once),
     // activations.
-    // table r is staged by wave r & (P - 1), P = largest power of two <= S
-    const int pmask = (1 << (31 - __builtin_clz(S))) - 1;
+    // wave s stages the tables of rows s, s + S, ...: with the usual eight waves for eight rows one each, found
+    // without a chain of per-row branches (whose address arithmetic would run for every row, ahead of the first load)
     const PairLane<BITS> pl = pair_lane<BITS>(lane);
+    const global_ptr<const half_t> lut_g = scalar_ptr(lut);
     TableWords<BITS> t[ROWS];
 #pragma unroll
-    for (int r = 0; r < ROWS; r++)
-        if (s == (r & pmask)) t[r] = lookup_table_fetch<BITS>(lut + (size_t)min(row0 + r, N - 1) * NC, lane, pl);
+    for (int i = 0; i < ROWS; i++) {
+        const int r = s + i * S;
+        if (r >= ROWS) break;
+        t[i] = lookup_table_fetch<BITS>(scalar_ptr(lut_g + (size_t)min(row0 + r, N - 1) * NC), lane, pl);
+    }
 
     uint32_t q[RQ][G][BITS];
     bool live[G];
@@ -127,11 +135,12 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     }
 
 #pragma unroll
-    for (int r = 0; r < ROWS; r++)
-        if (s == (r & pmask)) {
-            lookup_table_arrive<BITS>(t[r]);
-            lookup_table_stage<BITS>(t[r], tables[r], lane);
-        }
+    for (int i = 0; i < ROWS; i++) {
+        const int r = s + i * S;
+        if (r >= ROWS) break;
+        lookup_table_arrive<BITS>(t[i]);
+        lookup_table_stage<BITS>(t[i], tables[r], lane);
+    }
     if (S > 1) __syncthreads(); else __builtin_amdgcn_wave_barrier();
 
     // LDS byte address of this lane's table (LDS pointers are 32-bit offsets)
@@ -234,11 +243,12 @@ __global__ __launch_bounds__(THREADS) void gemv4_kbit_kernel(
     if (G > 1 || MG > 1 || (s * G + G) * 16 > W) compute(std::true_type{});
     else compute(std::false_type{});
     __syncthreads();
+    const global_ptr<half_t> out_g = (global_ptr<half_t>)reinterpret_cast<uint64_t>(out);  // a global store, not a flat one
     for (int o = s * kWave + lane; o < ROWS * MR; o += S * kWave) {
         const int m = o % MR, r = o / MR;
         float v = 0.f;
         for (int ss = 0; ss < S; ss++) v += partial[ss][r][m];
-        if (m < M && row0 + r < N) out[(size_t)m * N + row0 + r] = (half_t)v;
+        if (m < M && row0 + r < N) out_g[(size_t)m * N + row0 + r] = (half_t)v;
     }
 }
 

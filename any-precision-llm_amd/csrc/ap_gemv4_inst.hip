@@ -15,11 +15,11 @@ void launch_rq(const Gemv4Geometry &geo, const half_t *x, const uint32_t *qweigh
     const dim3 block(kWave, geo.S), grid(geo.grid);
     // smallest workgroup bound that holds S waves
     if (geo.S <= 4)
-        gemv4_kbit_kernel<BITS, MG, G, RQ, 256><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+        gemv4_kbit_kernel<BITS, MG, G, RQ, 256><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K, geo.S);
     else if (geo.S <= 8)
-        gemv4_kbit_kernel<BITS, MG, G, RQ, 512><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+        gemv4_kbit_kernel<BITS, MG, G, RQ, 512><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K, geo.S);
     else
-        gemv4_kbit_kernel<BITS, MG, G, RQ, 1024><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+        gemv4_kbit_kernel<BITS, MG, G, RQ, 1024><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K, geo.S);
 }
 
 template <int BITS>
@@ -39,9 +39,9 @@ void launch_two_groups(const Gemv4Geometry &geo, const half_t *x, const uint32_t
                        half_t *out, int M, int N, int K, hipStream_t stream) {
     const dim3 block(kWave, geo.S), grid(geo.grid);
     if (geo.S <= 4)
-        gemv4_kbit_kernel<BITS, 2, 1, 4, 256><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+        gemv4_kbit_kernel<BITS, 2, 1, 4, 256><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K, geo.S);
     else
-        gemv4_kbit_kernel<BITS, 2, 1, 4, 512><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K);
+        gemv4_kbit_kernel<BITS, 2, 1, 4, 512><<<grid, block, 0, stream>>>(x, qweight, lut, out, M, N, K, geo.S);
 }
 
 }  // namespace
