@@ -30,6 +30,7 @@
 #include "ap_gemm.hpp"
 #include "ap_gemmt_launch.hpp"
 #include "ap_lookup.hpp"
+#include "ap_reciprocal.hpp"
 
 namespace ap {
 
@@ -42,7 +43,8 @@ __device__ const uint32_t kGemmtZeros[64] = {};
 // and waves wait for each other's LDS round trips.
 template <int BITS, int RB, int MBW, int KH>
 __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(const half_t *__restrict__ x, const GemmtMembers mem,
-                                                                             int M, int K) {
+                                                                             int M, int K, int grid_m, uint32_t tile_div,
+                                                                             uint32_t tile_magic) {
     constexpr int NC = 1 << BITS;
     // 3 bits: the table of the weights of two adjacent elements (ap_lookup.hpp; 64 dword entries per row): half the table
     // reads, which are what loads the LDS port.  At 4 bits that table is 1 KB per row, 64 KB per workgroup: it pays where a CU
@@ -91,6 +93,17 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     const int wv = wave % kGemmtWaves, kh = wave / kGemmtWaves;  // row group of the wave, its half of K
     const int tid = wv * kWave + lane;                            // thread within the half
     const int col = lane & 15, grp = lane >> 4;
+    // Member 0 (the only one of a plain call) and the scalars every workgroup needs, named in ONE empty statement that
+    // wants them in scalar registers: one clause of scalar loads and one wait fetch them (the compiler alone loads an
+    // argument where it is first used -- here a chain of five dependent round trips to the scalar cache before the
+    // first plane load).  Pointers travel through it as integers and get their address space back afterwards.
+    static_assert(kGemmtMaxGroup == 4, "the member selection below is written out for four");
+    uint64_t x_i = reinterpret_cast<uint64_t>(x), q_i = reinterpret_cast<uint64_t>(mem.qweight[0]),
+             lut_i = reinterpret_cast<uint64_t>(mem.lut[0]), out_i = reinterpret_cast<uint64_t>(mem.out[0]);
+    int N0 = mem.N[0], count = mem.count, t1 = mem.tile0[1], t2 = mem.tile0[2], t3 = mem.tile0[3], t4 = mem.tile0[4];
+    long long ldo0 = mem.ldo[0];
+    asm volatile("" : "+s"(x_i), "+s"(q_i), "+s"(lut_i), "+s"(out_i), "+s"(N0), "+s"(count), "+s"(t1), "+s"(t2), "+s"(t3),
+                      "+s"(t4), "+s"(ldo0), "+s"(M), "+s"(K), "+s"(grid_m), "+s"(tile_div), "+s"(tile_magic));
     const int W = K >> 5;
     // Workgroup -> tile.  Consecutive workgroups go round-robin to the 8 XCDs, each with its own L2, and the tiles of
     // one block of weight rows over the activation rows read the same planes: they get workgroup numbers 8 apart, so
@@ -99,29 +112,43 @@ __global__ __launch_bounds__(kGemmtWaves *kWave *KH) void gemmt_kbit_kernel(cons
     // Beyond 8 tiles of activation rows the activations are the larger stream (16384 rows: 128 MB against 17 MB of
     // planes at 3 bits): there the weight-row tiles run fastest, so that the workgroups in flight share one tile of
     // activation rows in L2 (the other order measured 0.45 PFLOP/s against 0.70 there).
-    const int grid_m = (M + BM - 1) / BM, tiles_pad = (mem.tile0[mem.count] + 7) & ~7;
-    const int wg = blockIdx.x;
+    const int tiles = count <= 1 ? t1 : (count == 2 ? t2 : (count == 3 ? t3 : t4));  // tile0[count]
+    // grid_m = ceil(M / BM) and tile_div = 8 grid_m (up to 8 tiles of activation rows) or the padded number of
+    // weight-row tiles come from the host with tile_magic = reciprocal_floor(tile_div) (ap_reciprocal.hpp): the
+    // workgroup number is divided by one multiplication and a correction step.
+    uint32_t wq, wr;
+    divmod_by_reciprocal(blockIdx.x, tile_div, tile_magic, wq, wr);
     int tile_n, tile_m;
     if (grid_m <= 8) {
-        const int wa = wg / (8 * grid_m), wr = wg % (8 * grid_m);
-        tile_n = 8 * wa + (wr & 7);
-        tile_m = wr >> 3;
+        tile_n = 8 * (int)wq + (int)(wr & 7u);
+        tile_m = (int)(wr >> 3);
     } else {
-        tile_n = wg % tiles_pad;
-        tile_m = wg / tiles_pad;
+        tile_n = (int)wr;
+        tile_m = (int)wq;
     }
-    if (tile_n >= mem.tile0[mem.count]) return;  // padding (workgroup-uniform)
-    // the linear this tile belongs to (workgroup-uniform) and the tile's place in it
-    int g = 0;
-#pragma unroll
-    for (int i = 1; i < kGemmtMaxGroup; i++)
-        if (i < mem.count && tile_n >= mem.tile0[i]) g = i;
-    const uint32_t *__restrict__ qweight = mem.qweight[g];
-    const half_t *__restrict__ lut = reinterpret_cast<const half_t *>(mem.lut[g]);
-    half_t *__restrict__ out = reinterpret_cast<half_t *>(mem.out[g]);
-    const int N = mem.N[g];
-    const long long ldo = mem.ldo[g];
-    const int nb = (tile_n - mem.tile0[g]) * BN;  // first weight row of the workgroup
+    if (tile_n >= tiles) return;  // padding (workgroup-uniform)
+    // the linear this tile belongs to (workgroup-uniform) and the tile's place in it; a launch of several linears
+    // reads its member's fields by index (one more clause of scalar loads; a plain call skips it)
+    int N = N0, first_tile = 0;
+    long long ldo = ldo0;
+    if (count > 1) {
+        int g = tile_n >= t1 ? 1 : 0;  // tile0 ascends
+        g = (count > 2 && tile_n >= t2) ? 2 : g;
+        g = (count > 3 && tile_n >= t3) ? 3 : g;
+        if (g > 0) {
+            q_i = reinterpret_cast<uint64_t>(mem.qweight[g]);
+            lut_i = reinterpret_cast<uint64_t>(mem.lut[g]);
+            out_i = reinterpret_cast<uint64_t>(mem.out[g]);
+            N = mem.N[g];
+            ldo = mem.ldo[g];
+            first_tile = g == 1 ? t1 : (g == 2 ? t2 : t3);
+        }
+    }
+    x = (const half_t *)(global_ptr<const half_t>)x_i;
+    const uint32_t *__restrict__ qweight = (const uint32_t *)(global_ptr<const uint32_t>)q_i;
+    const half_t *__restrict__ lut = (const half_t *)(global_ptr<const half_t>)lut_i;
+    half_t *__restrict__ out = (half_t *)(global_ptr<half_t>)out_i;
+    const int nb = (tile_n - first_tile) * BN;  // first weight row of the workgroup
     const size_t plane_stride = (size_t)N * W;
     const int n0 = nb + wv * WROWS;     // ... of this wave
     const int m0 = tile_m * BM;         // first activation row of the tile
